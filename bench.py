@@ -1,0 +1,223 @@
+"""Benchmark of the fused batched-matmul path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others]
+
+One step = one pass of the hot path over one synthetic batch that is already
+resident in HBM.  The headline workload is the large fused min_bmm
+(A[1,65536,256] @ B[1,256,65536], min/argmin over dim=-1, product never
+stored); the JSON line also carries the roofline of its kernel, the same
+semantics timed with PyTorch on the host CPU, and short runs of the other
+configurations.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+PEAK_HBM_GBS = 8000.0
+
+
+def make_workloads(torch, cmk, dev):
+    """name -> dict(make=..., run=..., flop=..., desc=..., cpu=...)."""
+    def randn(*shape, seed):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        return torch.randn(*shape, generator=g, device=dev)
+
+    def rand_pm1(*shape, seed):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        return torch.rand(*shape, generator=g, device=dev) * 2 - 1
+
+    W = {}
+
+    def min_wl(name, M, N, K, cpu_rows):
+        op = cmk.MinBMMCUDA()
+
+        def make():
+            return randn(1, M, K, seed=0), randn(1, K, N, seed=1)
+
+        def cpu(A, B):   # torch.bmm(A, B).min(-1) on a slab of rows
+            return torch.bmm(A[:, :cpu_rows], B).min(-1)
+
+        W[name] = dict(make=make, run=lambda A, B: op(A, B, dim=-1), flop=2.0 * M * N * K,
+                       desc="min_bmm fp32 A[1,%d,%d] @ B[1,%d,%d], min+argmin over dim=-1" % (M, K, K, N),
+                       cpu=cpu, cpu_rows=cpu_rows, rows=M, cpu_flop_per_row=2.0 * N * K,
+                       cpu_expr="torch.bmm(A,B).min(-1)")
+
+    def topk_wl(name, M, N, K, cpu_rows):
+        op = cmk.TopkBMMCUDA()
+
+        def make():
+            return randn(1, M, K, seed=0), randn(1, K, N, seed=1)
+
+        def cpu(A, B):
+            return torch.bmm(A[:, :cpu_rows], B).topk(128, dim=-1)
+
+        W[name] = dict(make=make, run=lambda A, B: op(A, B, k=128, dim=-1), flop=2.0 * M * N * K,
+                       desc="topk_bmm fp32 A[1,%d,%d] @ B[1,%d,%d], k=128 over dim=-1" % (M, K, K, N),
+                       cpu=cpu, cpu_rows=cpu_rows, rows=M, cpu_flop_per_row=2.0 * N * K,
+                       cpu_expr="torch.bmm(A,B).topk(128,-1)")
+
+    def bmm_wl(name, L, M, N, K):
+        op = cmk.BMMCUDA()
+
+        def make():
+            return rand_pm1(L, M, K, seed=0), rand_pm1(L, K, N, seed=1)
+
+        W[name] = dict(make=make, run=lambda A, B: op(A, B), flop=2.0 * L * M * N * K,
+                       desc="bmm fp32 A[%d,%d,%d] @ B[%d,%d,%d]" % (L, M, K, L, K, N),
+                       bytes=4.0 * L * (M * N + M * K + K * N))
+
+    def mbmm_wl(name, L, M, N, K):
+        op = cmk.MBMMCUDA(share_mask=False)
+
+        def make():
+            A, B = randn(L, M, K, seed=0), randn(L, K, N, seed=1)
+            g = torch.Generator().manual_seed(1)
+            tiles = torch.rand(L, M // 128, N // 128, generator=g) < 0.5
+            keep = tiles.repeat_interleave(128, 1).repeat_interleave(128, 2)
+            fm = torch.tril(torch.ones(M, N)).bool()[None] & keep
+            bm, tm, em = cmk.derive_masks(fm)
+            kept_tiles = int(bm.sum())
+            return A, B, bm.to(dev), tm.to(dev), em.to(dev), kept_tiles
+
+        W[name] = dict(make=make, run=lambda A, B, bm, tm, em, kt: op(A, B, bm, tm, em),
+                       flop=2.0 * L * M * N * K,
+                       desc="mbmm fp32 A[%d,%d,%d] @ B[%d,%d,%d], tril & tile-Bernoulli(0.5) mask" % (L, M, K, L, K, N),
+                       bytes=4.0 * L * (M * N + M * K + K * N) + L * M * N + L * (M // 8) * (N // 8))
+
+    min_wl("min_bmm_large", 65536, 65536, 256, cpu_rows=4096)
+    min_wl("min_bmm_small", 4096, 4096, 64, cpu_rows=4096)
+    topk_wl("topk_bmm", 1048576, 1024, 256, cpu_rows=65536)
+    bmm_wl("bmm", 128, 1024, 1024, 128)
+    mbmm_wl("mbmm", 128, 1024, 1024, 64)
+    return W
+
+
+def time_steps(torch, fn, steps, warmup):
+    """Wall time of exactly `steps` steps between synchronisations, plus the
+    per-launch device time from events recorded on the launch stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for s in range(steps):
+        starts[s].record()
+        fn()
+        ends[s].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = [starts[s].elapsed_time(ends[s]) for s in range(steps)]
+    return wall, dev_ms
+
+
+def cpu_baseline(torch, wl, args_dev, budget_s=12.0):
+    """The reference semantics with PyTorch on the host cores, on a bounded
+    sample (slabs of rows of the same workload)."""
+    if "cpu" not in wl:
+        return None
+    A, B = args_dev[0].cpu(), args_dev[1].cpu()
+    torch.set_num_threads(os.cpu_count() or 1)
+    wl["cpu"](A, B)                                  # warm-up slab
+    done_rows, t_total = 0, 0.0
+    rows = wl["cpu_rows"]
+    off = 0
+    while t_total < budget_s and off + rows <= wl["rows"] and done_rows < 4 * rows:
+        a = A[:, off:off + rows]
+        t0 = time.perf_counter()
+        wl["cpu"](a, B)
+        t_total += time.perf_counter() - t0
+        done_rows += rows
+        off += rows
+    gflops = done_rows * wl["cpu_flop_per_row"] / t_total / 1e9
+    return {"value": round(gflops, 2), "unit": "GFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": "%s on %d of %d rows, %d threads, %.2f s" % (
+                wl["cpu_expr"], done_rows, wl["rows"], torch.get_num_threads(), t_total)}
+
+
+def run_workload(torch, wl, steps, warmup):
+    args = wl["make"]()
+    torch.cuda.synchronize()
+    wall, dev_ms = time_steps(torch, lambda: wl["run"](*args), steps, warmup)
+    ms = wall * 1e3 / steps
+    kern_ms = statistics.mean(dev_ms)
+    return args, ms, kern_ms
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="min_bmm_large")
+    ap.add_argument("--no-others", action="store_true", help="skip the short runs of the other configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported "
+              "(every output row depends on one row of A and all of B, so the path "
+              "shards by rows without communication; see DESIGN.md)" % a.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import custom_matmul_kernels_amd as cmk
+    cmk.load()                                       # fails loudly if libcmk.so is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    W = make_workloads(torch, cmk, dev)
+    wl = W[a.workload]
+
+    args, ms, kern_ms = run_workload(torch, wl, a.steps, a.warmup)
+    gflops = wl["flop"] / (ms * 1e-3) / 1e9
+    achieved = wl["flop"] / (kern_ms * 1e-3) / 1e12
+    out = {
+        "metric": "GFLOP/s of fused %s (2*M*N*K / time), fp32 MFMA" % a.workload.split("_large")[0].split("_small")[0],
+        "value": round(gflops, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": wl["desc"], "name": a.workload},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                     "traffic": None, "kernel_ms": round(kern_ms, 4)},
+    }
+    if not a.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(torch, wl, args)
+    del args
+    torch.cuda.empty_cache()
+
+    if not a.no_others:
+        others = {}
+        for name, w in W.items():
+            if name == a.workload:
+                continue
+            steps = 5 if name == "topk_bmm" else 20
+            args, ms_o, kern_o = run_workload(torch, w, steps, 3)
+            rec = {"workload": w["desc"], "ms_per_step": round(ms_o, 4), "kernel_ms": round(kern_o, 4),
+                   "GFLOP/s": round(w["flop"] / (kern_o * 1e-3) / 1e9, 1),
+                   "frac_fp32_mfma_peak": round(w["flop"] / (kern_o * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
+            if "bytes" in w:
+                rec["GB/s"] = round(w["bytes"] / (kern_o * 1e-3) / 1e9, 1)
+                rec["frac_hbm_peak"] = round(rec["GB/s"] / PEAK_HBM_GBS, 4)
+            if name == "mbmm":
+                kept = args[5]
+                rec["kept_tiles"] = kept
+                rec["executed_GFLOP/s"] = round(2.0 * 128 * 128 * 64 * kept / (kern_o * 1e-3) / 1e9, 1)
+            if not a.no_cpu and "cpu" in w and name != "min_bmm_small":
+                rec["cpu_baseline"] = cpu_baseline(torch, w, args, budget_s=6.0)
+            others[name] = rec
+            del args
+            torch.cuda.empty_cache()
+        out["other_workloads"] = others
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,185 @@
+// bmm / mbmm: dense and masked batched product with a store epilogue.
+//
+// X = the m side (rows of C, inside a lane), Y = the n side (columns of C,
+// across lanes): a store of one accumulator register writes two 128-byte row
+// segments of C.  One work-group = one 128x128 tile of C, which is also the
+// granularity of the block mask (reference kernels/mbmm.cu:247-255).
+#include "cmk_core.hpp"
+#include "cmk_launch.hpp"
+
+namespace cmk {
+
+struct BmmArgs {
+  const float* A;
+  const float* B;
+  float* C;
+  const uint8_t* block_mask;
+  const uint8_t* thread_mask;
+  const uint8_t* element_mask;
+  long long lda, ldb, strideA, strideB;
+  int L, M, N, K;
+  int tiles_m, tiles_n, group_m;
+  int mask_batched;  // 1: masks have a leading batch axis, 0: shared by all batches
+  int vecA, vecB;
+};
+
+template <int XK, int YK, bool MASKED>
+__global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
+  using C = Core<XK, YK, 2, 2, 2, 2>;
+  __shared__ __attribute__((aligned(16))) float lds[C::ldsFloats];
+
+  const int tiles = a.tiles_m * a.tiles_n;
+  const int logical = xcd_logical_id(blockIdx.x, a.L * tiles);
+  if (logical < 0) return;
+  const int b = logical / tiles;
+  const int t = logical - b * tiles;
+  // grouped rasterisation: walk group_m tile-rows together so that concurrently
+  // running work-groups share panels of A and B in L2
+  const int per_group = a.group_m * a.tiles_n;
+  const int g = t / per_group;
+  const int first_m = g * a.group_m;
+  const int gsz = min(a.tiles_m - first_m, a.group_m);
+  const int in_g = t - g * per_group;
+  const int tile_m = first_m + in_g % gsz;
+  const int tile_n = in_g / gsz;
+  const int m0 = tile_m * C::TX;
+  const int n0 = tile_n * C::TY;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int l32 = lane & 31;
+  const int half = lane >> 5;
+  float* Cb = a.C + (long long)b * a.M * a.N;
+
+  long long mb = 0;  // batch index into the masks
+  if constexpr (MASKED) {
+    mb = a.mask_batched ? b : 0;
+    const uint8_t bm = a.block_mask[(mb * a.tiles_m + tile_m) * a.tiles_n + tile_n];
+    if (bm == 0) {
+      // skipped tile: nothing is loaded or multiplied, zeros are written
+      for (int e = threadIdx.x; e < 128 * 32; e += kThreads) {
+        const int r = m0 + (e >> 5);
+        const int c = n0 + (e & 31) * 4;
+        if (r < a.M) {
+          float* dst = Cb + (long long)r * a.N + c;
+          if ((a.N & 3) == 0 && c + 3 < a.N) {
+            *reinterpret_cast<f32x4*>(dst) = f32x4{0.f, 0.f, 0.f, 0.f};
+          } else {
+            for (int j = 0; j < 4; ++j)
+              if (c + j < a.N) dst[j] = 0.f;
+          }
+        }
+      }
+      return;
+    }
+  }
+
+  Operand X{a.A + (long long)b * a.strideA, a.lda, a.M, a.vecA};
+  Operand Y{a.B + (long long)b * a.strideB, a.ldb, a.N, a.vecB};
+
+  C core;
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int S = max(1, (a.K + KS - 1) / KS);
+  core.load(X, Y, m0, n0, 0, a.K);
+  core.store(lds);
+  __syncthreads();
+  for (int s = 0; s < S; ++s) {
+    const bool more = s + 1 < S;
+    if (more) core.load(X, Y, m0, n0, (s + 1) * KS, a.K);
+    core.mma(lds + (s & 1) * C::bufFloats, acc);
+    if (more) core.store(lds + ((s + 1) & 1) * C::bufFloats);
+    __syncthreads();
+  }
+
+  // epilogue
+  const int mw = m0 + (wave % 2) * 64;
+  const int nw = n0 + (wave / 2) * 64;
+#pragma unroll
+  for (int bx = 0; bx < 2; ++bx) {
+#pragma unroll
+    for (int by = 0; by < 2; ++by) {
+      const int n = nw + by * 32 + l32;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = mw + bx * 32 + acc_row(r, half);
+        if (m < a.M && n < a.N) {
+          float v = acc[bx][by][r];
+          if constexpr (MASKED) {
+            const int tn8 = (a.N + 7) >> 3;
+            const int tm8 = (a.M + 7) >> 3;
+            const uint8_t tm = a.thread_mask[(mb * tm8 + (m >> 3)) * tn8 + (n >> 3)];
+            const uint8_t em = a.element_mask[(mb * a.M + m) * a.N + n];
+            v = tm ? v * (float)em : 0.f;
+          }
+          Cb[(long long)m * a.N + n] = v;
+        }
+      }
+    }
+  }
+}
+
+template <bool MASKED>
+static hipError_t launch_bmm(const BmmArgs& a, int transA, int transB, hipStream_t st) {
+  const int total = a.L * a.tiles_m * a.tiles_n;
+  const dim3 grid(((total + 7) / 8) * 8), block(kThreads);
+  // A "n" is k-contiguous (KC), A "t" is m-contiguous (RC);
+  // B "n" is n-contiguous (RC), B "t" is k-contiguous (KC).
+  if (!transA && !transB) hipLaunchKernelGGL((bmm_kernel<KC, RC, MASKED>), grid, block, 0, st, a);
+  else if (!transA && transB) hipLaunchKernelGGL((bmm_kernel<KC, KC, MASKED>), grid, block, 0, st, a);
+  else if (transA && !transB) hipLaunchKernelGGL((bmm_kernel<RC, RC, MASKED>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((bmm_kernel<RC, KC, MASKED>), grid, block, 0, st, a);
+  return hipGetLastError();
+}
+
+static BmmArgs make_args(const float* A, const float* B, float* C, const cmk_gemm_desc* d) {
+  BmmArgs a{};
+  a.A = A; a.B = B; a.C = C;
+  a.lda = d->lda; a.ldb = d->ldb; a.strideA = d->strideA; a.strideB = d->strideB;
+  a.L = d->L; a.M = d->M; a.N = d->N; a.K = d->K;
+  a.tiles_m = (d->M + 127) / 128;
+  a.tiles_n = (d->N + 127) / 128;
+  a.group_m = 4;
+  a.vecA = vec_ok(A, d->lda, d->strideA);
+  a.vecB = vec_ok(B, d->ldb, d->strideB);
+  return a;
+}
+
+}  // namespace cmk
+
+using namespace cmk;
+
+extern "C" int cmk_bmm_f32(const float* A, const float* B, float* C, const cmk_gemm_desc* d,
+                           void* stream) {
+  if (int e = check_desc(d)) return e;
+  if (d->L == 0 || d->M == 0 || d->N == 0) return CMK_OK;
+  if (!A || !B || !C) return fail(CMK_ERR_INVALID_ARG, "cmk_bmm_f32: null pointer");
+  if (int e = check_grid((long long)d->L * ((d->M + 127) / 128) * ((d->N + 127) / 128))) return e;
+  BmmArgs a = make_args(A, B, C, d);
+  return hip_status(launch_bmm<false>(a, d->transA, d->transB, (hipStream_t)stream),
+                    "cmk_bmm_f32 launch");
+}
+
+extern "C" int cmk_mbmm_f32(const float* A, const float* B, float* C, const uint8_t* block_mask,
+                            const uint8_t* thread_mask, const uint8_t* element_mask,
+                            int share_mask, const cmk_gemm_desc* d, void* stream) {
+  if (int e = check_desc(d)) return e;
+  if (d->transA || d->transB)
+    return fail(CMK_ERR_UNSUPPORTED, "cmk_mbmm_f32: only the \"nn\" layout is implemented");
+  if (d->L == 0 || d->M == 0 || d->N == 0) return CMK_OK;
+  if (!A || !B || !C || !block_mask || !thread_mask || !element_mask)
+    return fail(CMK_ERR_INVALID_ARG, "cmk_mbmm_f32: null pointer");
+  if (int e = check_grid((long long)d->L * ((d->M + 127) / 128) * ((d->N + 127) / 128))) return e;
+  BmmArgs a = make_args(A, B, C, d);
+  a.block_mask = block_mask;
+  a.thread_mask = thread_mask;
+  a.element_mask = element_mask;
+  a.mask_batched = share_mask ? 0 : 1;
+  return hip_status(launch_bmm<true>(a, 0, 0, (hipStream_t)stream), "cmk_mbmm_f32 launch");
+}

@@ -1,0 +1,217 @@
+// Shared fp32-MFMA tiled GEMM core for gfx950 (CDNA4, wave64).
+//
+// One 256-thread work-group (4 waves) computes a TX x TY macro tile of the
+// product of two operands that both have a contraction axis k:
+//   X : TX "rows"  -> MFMA source A, the axis that ends up INSIDE a lane
+//   Y : TY "rows"  -> MFMA source B, the axis that ends up ACROSS lanes
+// Which matrix of the user's problem plays X and which plays Y is chosen by
+// each kernel so that its epilogue is cheap: a reduction wants the reduced
+// axis in X (running state stays in one lane), a row-major store wants the
+// contiguous axis in Y (a store instruction writes 128-byte row segments).
+//
+// The contraction is walked in slabs of KS = 32.  A slab of each operand is
+// fetched from global memory into registers, written to one of two LDS
+// buffers, and consumed from the other with v_mfma_f32_32x32x2_f32.  Inside a
+// slab, k is consumed in groups of 8: lanes 0-31 feed k = 8g+0..3 and lanes
+// 32-63 feed k = 8g+4..7 of both operands, so one 128-bit LDS read per 32x32
+// block supplies four MFMA steps.  (A sum over k does not care about the
+// order, as long as both operands use the same one.)
+//
+// An operand tile can sit in memory, and in LDS, in one of two ways:
+//   KC : element(row, k) at row*ld + k   (k contiguous)  -> LDS [row][KS+4]
+//   RC : element(row, k) at k*ld + row   (rows contiguous) -> LDS [k][T+8]
+// Both are written with 128-bit stores straight from 128-bit global loads;
+// no transposition is needed on the way in.
+//
+// Plays the role of load_ab_*, buffer2smem_* and thread_matmul_* of the
+// reference (kernels/bmm_helpers.cu:114-164, 240-622).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace cmk {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int KS = 32;  // contraction depth of one LDS slab
+constexpr int KC = 0;   // k-contiguous operand
+constexpr int RC = 1;   // row-contiguous operand
+
+struct Operand {
+  const float* p;  // base of this batch's matrix
+  long long ld;    // KC: distance between rows; RC: distance between k
+  int rows;        // extent of the non-contracted axis
+  int vec;         // non-zero when 16-byte loads are legal (base and ld aligned)
+};
+
+template <int KIND, int T>
+struct TileLayout;
+template <int T>
+struct TileLayout<KC, T> {
+  static constexpr int pitch = KS + 4;
+  static constexpr int floats = T * pitch;
+};
+template <int T>
+struct TileLayout<RC, T> {
+  static constexpr int pitch = T + 8;
+  static constexpr int floats = KS * pitch;
+};
+
+// ---- global -> registers ---------------------------------------------------
+template <int KIND, int T>
+__device__ __forceinline__ void gload(const Operand& o, int r0, int k0, int K,
+                                      f32x4 (&v)[T / 32]) {
+  const int t = threadIdx.x;
+  if constexpr (KIND == KC) {
+    const int kk = k0 + (t & 7) * 4;
+    const int rr = r0 + (t >> 3);
+#pragma unroll
+    for (int p = 0; p < T / 32; ++p) {
+      const int row = rr + 32 * p;
+      f32x4 val = {0.f, 0.f, 0.f, 0.f};
+      if (row < o.rows) {
+        const float* src = o.p + (long long)row * o.ld + kk;
+        if (o.vec && kk + 3 < K) {
+          val = *reinterpret_cast<const f32x4*>(src);
+        } else {
+          if (kk + 0 < K) val.x = src[0];
+          if (kk + 1 < K) val.y = src[1];
+          if (kk + 2 < K) val.z = src[2];
+          if (kk + 3 < K) val.w = src[3];
+        }
+      }
+      v[p] = val;
+    }
+  } else {
+    constexpr int TPR = T / 4;           // threads per k-row
+    constexpr int RPP = kThreads / TPR;  // k-rows per pass
+    const int rr = r0 + (t % TPR) * 4;
+    const int kb = k0 + t / TPR;
+#pragma unroll
+    for (int p = 0; p < T / 32; ++p) {
+      const int kk = kb + p * RPP;
+      f32x4 val = {0.f, 0.f, 0.f, 0.f};
+      if (kk < K) {
+        const float* src = o.p + (long long)kk * o.ld + rr;
+        if (o.vec && rr + 3 < o.rows) {
+          val = *reinterpret_cast<const f32x4*>(src);
+        } else {
+          if (rr + 0 < o.rows) val.x = src[0];
+          if (rr + 1 < o.rows) val.y = src[1];
+          if (rr + 2 < o.rows) val.z = src[2];
+          if (rr + 3 < o.rows) val.w = src[3];
+        }
+      }
+      v[p] = val;
+    }
+  }
+}
+
+// ---- registers -> LDS --------------------------------------------------------
+template <int KIND, int T>
+__device__ __forceinline__ void lstore(float* lds, const f32x4 (&v)[T / 32]) {
+  const int t = threadIdx.x;
+  constexpr int pitch = TileLayout<KIND, T>::pitch;
+  if constexpr (KIND == KC) {
+#pragma unroll
+    for (int p = 0; p < T / 32; ++p)
+      *reinterpret_cast<f32x4*>(&lds[((t >> 3) + 32 * p) * pitch + (t & 7) * 4]) = v[p];
+  } else {
+    constexpr int TPR = T / 4;
+    constexpr int RPP = kThreads / TPR;
+#pragma unroll
+    for (int p = 0; p < T / 32; ++p)
+      *reinterpret_cast<f32x4*>(&lds[(t / TPR + p * RPP) * pitch + (t % TPR) * 4]) = v[p];
+  }
+}
+
+// ---- LDS -> MFMA fragment ----------------------------------------------------
+// Four k values (8*kg + 4*half + 0..3) of tile row `row` for this lane.
+template <int KIND, int T>
+__device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg, int half) {
+  constexpr int pitch = TileLayout<KIND, T>::pitch;
+  if constexpr (KIND == KC) {
+    return *reinterpret_cast<const f32x4*>(&lds[row * pitch + kg * 8 + half * 4]);
+  } else {
+    const float* q = &lds[(kg * 8 + half * 4) * pitch + row];
+    f32x4 r;
+    r.x = q[0];
+    r.y = q[pitch];
+    r.z = q[2 * pitch];
+    r.w = q[3 * pitch];
+    return r;
+  }
+}
+
+// Work-group level tile engine.  WX x WY waves (WX*WY == 4), each wave owns
+// BX x BY blocks of 32x32.
+template <int XK, int YK, int WX, int WY, int BX, int BY>
+struct Core {
+  static_assert(WX * WY == 4, "four waves per work-group");
+  static constexpr int TX = WX * BX * 32;
+  static constexpr int TY = WY * BY * 32;
+  static constexpr int xFloats = TileLayout<XK, TX>::floats;
+  static constexpr int yFloats = TileLayout<YK, TY>::floats;
+  static constexpr int bufFloats = xFloats + yFloats;
+  static constexpr int ldsFloats = 2 * bufFloats;
+
+  f32x4 xv[TX / 32];
+  f32x4 yv[TY / 32];
+
+  __device__ __forceinline__ void load(const Operand& X, const Operand& Y, int x0, int y0,
+                                       int k0, int K) {
+    gload<XK, TX>(X, x0, k0, K, xv);
+    gload<YK, TY>(Y, y0, k0, K, yv);
+  }
+  __device__ __forceinline__ void store(float* buf) {
+    lstore<XK, TX>(buf, xv);
+    lstore<YK, TY>(buf + xFloats, yv);
+  }
+  // acc[bx][by] += X-block(bx) * Y-block(by) over the slab held in `buf`.
+  __device__ __forceinline__ void mma(const float* buf, f32x16 (&acc)[BX][BY]) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+    const int xr = (wave % WX) * BX * 32 + l32;
+    const int yr = (wave / WX) * BY * 32 + l32;
+    const float* bx_ = buf;
+    const float* by_ = buf + xFloats;
+#pragma unroll
+    for (int kg = 0; kg < KS / 8; ++kg) {
+      f32x4 xf[BX], yf[BY];
+#pragma unroll
+      for (int b = 0; b < BX; ++b) xf[b] = frag<XK, TX>(bx_, xr + 32 * b, kg, half);
+#pragma unroll
+      for (int b = 0; b < BY; ++b) yf[b] = frag<YK, TY>(by_, yr + 32 * b, kg, half);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int bx = 0; bx < BX; ++bx)
+#pragma unroll
+          for (int by = 0; by < BY; ++by)
+            acc[bx][by] =
+                __builtin_amdgcn_mfma_f32_32x32x2f32(xf[bx][j], yf[by][j], acc[bx][by], 0, 0, 0);
+    }
+  }
+};
+
+// Element (bx, by, r) of a wave's accumulators sits at
+//   x = wave_x*BX*32 + bx*32 + acc_row(r, half),   y = wave_y*BY*32 + by*32 + lane%32.
+__device__ __forceinline__ int acc_row(int r, int half) {
+  return 8 * (r >> 2) + 4 * half + (r & 3);
+}
+
+// Work-group ids are dealt round-robin to the 8 XCDs (each with a private
+// L2).  This maps the hardware id to a logical id such that every XCD walks a
+// contiguous range of logical ids; `per` = ceil(total / 8) and the grid is
+// launched with 8*per work-groups.  Returns -1 for the padding ids.
+__device__ __forceinline__ int xcd_logical_id(int hw_id, int total) {
+  const int per = (total + 7) >> 3;
+  const int logical = (hw_id & 7) * per + (hw_id >> 3);
+  return logical < total ? logical : -1;
+}
+
+}  // namespace cmk

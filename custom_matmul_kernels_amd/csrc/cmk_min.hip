@@ -1,0 +1,262 @@
+// min_bmm: fused min / argmin of A@B along one axis; the product never
+// reaches HBM.
+//
+// X = the reduced axis, Y = the kept axis.  With X inside the lane, the
+// running (min, argmin) of an output element lives in one lane for the whole
+// walk over X; the finish is one exchange between the two half-waves and one
+// LDS step between the two waves that share a Y range.  When the kept axis
+// has too few 128-wide strips to fill the chip, the reduced axis is also cut
+// into `splits` ranges; their partial results go to a workspace and a small
+// second kernel folds them in order, so ties always resolve to the lowest
+// index and the result does not depend on scheduling.
+//
+// Plays the role of min_bmm_* with min_dim_1 / min_dim_2 and the float
+// atomicMin (reference kernels/minbmm.cu:1-153, 347-440).
+#include <math.h>
+
+#include "cmk_core.hpp"
+#include "cmk_launch.hpp"
+
+namespace cmk {
+
+struct MinArgs {
+  Operand X, Y;                 // batch 0 views
+  long long strideX, strideY;   // batch strides
+  float* values;                // [L][Yext]
+  long long* indices;           // [L][Yext]
+  float* part_val;              // [splits][L][Yext]  (splits > 1)
+  int* part_idx;
+  int L, K;
+  int ystrips, xtiles, splits, tiles_per_split;
+};
+
+template <int XK, int YK>
+__global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
+  using C = Core<XK, YK, 2, 2, 2, 2>;
+  __shared__ __attribute__((aligned(16))) float lds[C::ldsFloats];
+
+  const int total = a.L * a.ystrips * a.splits;
+  const int logical = xcd_logical_id(blockIdx.x, total);
+  if (logical < 0) return;
+  // split is the slowest index: work-groups that run together walk the same
+  // range of X and share its tiles in L2
+  const int split = logical / (a.L * a.ystrips);
+  const int rem = logical - split * (a.L * a.ystrips);
+  const int b = rem / a.ystrips;
+  const int ystrip = rem - b * a.ystrips;
+  const int y0 = ystrip * C::TY;
+  const int xt_begin = split * a.tiles_per_split;
+  const int xt_end = min(a.xtiles, xt_begin + a.tiles_per_split);
+
+  Operand X = a.X, Y = a.Y;
+  X.p += (long long)b * a.strideX;
+  Y.p += (long long)b * a.strideY;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int l32 = lane & 31;
+  const int half = lane >> 5;
+  const int wx = wave % 2, wy = wave / 2;
+
+  float best[2] = {INFINITY, INFINITY};
+  int bidx[2] = {xt_begin * C::TX, xt_begin * C::TX};
+
+  C core;
+  const int S = max(1, (a.K + KS - 1) / KS);
+  const int iters = (xt_end - xt_begin) * S;
+  if (iters > 0) {
+    core.load(X, Y, xt_begin * C::TX, y0, 0, a.K);
+    core.store(lds);
+  }
+  __syncthreads();
+  int it = 0;
+  for (int xt = xt_begin; xt < xt_end; ++xt) {
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int s = 0; s < S; ++s, ++it) {
+      const bool more = it + 1 < iters;
+      if (more) {
+        const bool wrap = (s + 1 == S);
+        core.load(X, Y, (wrap ? xt + 1 : xt) * C::TX, y0, wrap ? 0 : (s + 1) * KS, a.K);
+      }
+      core.mma(lds + (it & 1) * C::bufFloats, acc);
+      if (s == S - 1) {
+        // fold this tile into the running minimum; indices ascend within a
+        // lane, so a strict '<' keeps the first occurrence
+        const int xb = xt * C::TX + wx * 64;
+        if (xb + 64 <= X.rows) {
+#pragma unroll
+          for (int bx = 0; bx < 2; ++bx)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int x = xb + bx * 32 + acc_row(r, half);
+#pragma unroll
+              for (int by = 0; by < 2; ++by) {
+                const float v = acc[bx][by][r];
+                if (v < best[by]) { best[by] = v; bidx[by] = x; }
+              }
+            }
+        } else {
+#pragma unroll
+          for (int bx = 0; bx < 2; ++bx)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int x = xb + bx * 32 + acc_row(r, half);
+#pragma unroll
+              for (int by = 0; by < 2; ++by) {
+                const float v = acc[bx][by][r];
+                if (x < X.rows && v < best[by]) { best[by] = v; bidx[by] = x; }
+              }
+            }
+        }
+      }
+      if (more) core.store(lds + ((it + 1) & 1) * C::bufFloats);
+      __syncthreads();
+    }
+  }
+
+  // the two half-waves hold different x for the same y
+#pragma unroll
+  for (int by = 0; by < 2; ++by) {
+    const float ov = __shfl_xor(best[by], 32);
+    const int oi = __shfl_xor(bidx[by], 32);
+    if (ov < best[by] || (ov == best[by] && oi < bidx[by])) { best[by] = ov; bidx[by] = oi; }
+  }
+  // the two waves with the same wy hold different x for the same y
+  float* red_v = lds;                                   // [2 wy][2 by][32]
+  int* red_i = reinterpret_cast<int*>(lds + 128);
+  if (wx == 1 && half == 0) {
+#pragma unroll
+    for (int by = 0; by < 2; ++by) {
+      red_v[(wy * 2 + by) * 32 + l32] = best[by];
+      red_i[(wy * 2 + by) * 32 + l32] = bidx[by];
+    }
+  }
+  __syncthreads();
+  if (wx == 0 && half == 0) {
+    const int Yext = Y.rows;
+#pragma unroll
+    for (int by = 0; by < 2; ++by) {
+      const float ov = red_v[(wy * 2 + by) * 32 + l32];
+      const int oi = red_i[(wy * 2 + by) * 32 + l32];
+      float v = best[by];
+      int i = bidx[by];
+      if (ov < v || (ov == v && oi < i)) { v = ov; i = oi; }
+      const int y = y0 + wy * 64 + by * 32 + l32;
+      if (y < Yext) {
+        if (a.splits == 1) {
+          a.values[(long long)b * Yext + y] = v;
+          a.indices[(long long)b * Yext + y] = i;
+        } else {
+          const long long o = ((long long)split * a.L + b) * Yext + y;
+          a.part_val[o] = v;
+          a.part_idx[o] = i;
+        }
+      }
+    }
+  }
+}
+
+// Folds the per-split partial results in ascending split (= ascending index)
+// order.
+__global__ void min_fold_kernel(const float* part_val, const int* part_idx, float* values,
+                                long long* indices, long long rows, int splits) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows) return;
+  float v = part_val[i];
+  int idx = part_idx[i];
+  for (int s = 1; s < splits; ++s) {
+    const float ov = part_val[(long long)s * rows + i];
+    if (ov < v) { v = ov; idx = part_idx[(long long)s * rows + i]; }
+  }
+  values[i] = v;
+  indices[i] = idx;
+}
+
+// How the reduced axis is cut: enough work-groups to give every CU a couple,
+// never more splits than tiles.
+static void plan_min(int L, int Xext, int Yext, int* ystrips, int* xtiles, int* splits,
+                     int* tiles_per_split) {
+  *ystrips = ceil_div(Yext, 128);
+  *xtiles = ceil_div(Xext, 128);
+  const long long strips = (long long)L * *ystrips;
+  int want = 1;
+  if (strips < 512) want = (int)((512 + strips - 1) / strips);
+  if (want > *xtiles) want = *xtiles;
+  if (want < 1) want = 1;
+  *tiles_per_split = ceil_div(*xtiles, want);
+  *splits = ceil_div(*xtiles, *tiles_per_split);
+}
+
+size_t min_workspace_bytes(int L, int Xext, int Yext) {
+  int ys, xt, sp, tps;
+  plan_min(L, Xext, Yext, &ys, &xt, &sp, &tps);
+  if (sp <= 1) return 0;
+  return (size_t)sp * L * Yext * 8;
+}
+
+}  // namespace cmk
+
+using namespace cmk;
+
+extern "C" int cmk_min_bmm_f32(const float* A, const float* B, float* values, long long* indices,
+                               const cmk_gemm_desc* d, int dim, int distance, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+  if (int e = check_desc(d)) return e;
+  if (dim != 1 && dim != 2) return fail(CMK_ERR_INVALID_ARG, "cmk_min_bmm_f32: dim must be 1 or 2");
+  if (distance < CMK_DIST_INNER || distance > CMK_DIST_L1)
+    return fail(CMK_ERR_INVALID_ARG, "cmk_min_bmm_f32: unknown distance %d", distance);
+  if (distance != CMK_DIST_INNER)
+    return fail(CMK_ERR_UNSUPPORTED, "cmk_min_bmm_f32: only distance \"inner\" is implemented");
+  const int Xext = dim == 2 ? d->N : d->M;
+  const int Yext = dim == 2 ? d->M : d->N;
+  if (Xext == 0) return fail(CMK_ERR_INVALID_ARG, "cmk_min_bmm_f32: reduction over an empty axis");
+  if (d->L == 0 || Yext == 0) return CMK_OK;
+  if (!values || !indices || (d->K > 0 && (!A || !B)))
+    return fail(CMK_ERR_INVALID_ARG, "cmk_min_bmm_f32: null pointer");
+
+  MinArgs a{};
+  // operand kinds: A "n" is k-contiguous, A "t" is m-contiguous; B "n" is
+  // n-contiguous, B "t" is k-contiguous
+  const Operand opA{A, d->lda, d->M, vec_ok(A, d->lda, d->strideA)};
+  const Operand opB{B, d->ldb, d->N, vec_ok(B, d->ldb, d->strideB)};
+  const int kindA = d->transA ? RC : KC;
+  const int kindB = d->transB ? KC : RC;
+  int xk, yk;
+  if (dim == 2) { a.X = opB; a.Y = opA; a.strideX = d->strideB; a.strideY = d->strideA; xk = kindB; yk = kindA; }
+  else          { a.X = opA; a.Y = opB; a.strideX = d->strideA; a.strideY = d->strideB; xk = kindA; yk = kindB; }
+  a.values = values;
+  a.indices = indices;
+  a.L = d->L;
+  a.K = d->K;
+  plan_min(d->L, Xext, Yext, &a.ystrips, &a.xtiles, &a.splits, &a.tiles_per_split);
+  if (a.splits > 1) {
+    const size_t need = (size_t)a.splits * d->L * Yext * 8;
+    if (!workspace || workspace_bytes < need)
+      return fail(CMK_ERR_WORKSPACE, "cmk_min_bmm_f32: workspace of %zu bytes required, %zu given",
+                  need, workspace_bytes);
+    a.part_val = static_cast<float*>(workspace);
+    a.part_idx = reinterpret_cast<int*>(a.part_val + (size_t)a.splits * d->L * Yext);
+  }
+  const long long total = (long long)d->L * a.ystrips * a.splits;
+  if (int e = check_grid(total)) return e;
+  const dim3 grid((unsigned)(((total + 7) / 8) * 8)), block(kThreads);
+  hipStream_t st = (hipStream_t)stream;
+  if (xk == KC && yk == KC) hipLaunchKernelGGL((min_kernel<KC, KC>), grid, block, 0, st, a);
+  else if (xk == KC && yk == RC) hipLaunchKernelGGL((min_kernel<KC, RC>), grid, block, 0, st, a);
+  else if (xk == RC && yk == KC) hipLaunchKernelGGL((min_kernel<RC, KC>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((min_kernel<RC, RC>), grid, block, 0, st, a);
+  if (int e = hip_status(hipGetLastError(), "cmk_min_bmm_f32 launch")) return e;
+  if (a.splits > 1) {
+    const long long rows = (long long)d->L * Yext;
+    hipLaunchKernelGGL(min_fold_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st,
+                       a.part_val, a.part_idx, values, indices, rows, a.splits);
+    if (int e = hip_status(hipGetLastError(), "cmk_min_bmm_f32 fold launch")) return e;
+  }
+  return CMK_OK;
+}

@@ -1,0 +1,368 @@
+// topk_bmm: fused per-row top-128 (largest, sorted descending) of A@B along
+// one axis; the product never reaches HBM.
+//
+// X = the reduced axis (inside a lane), Y = the kept axis.  A work-group owns a
+// strip of 32 complete output rows and walks the reduced axis in chunks of
+// 1024 candidates (8 tiles of 128) whose accumulators all stay in registers.
+// After each chunk the accumulators go through LDS, eight rows at a time, so
+// that one wave sees one row's 1024 candidates (16 per lane) together with the
+// row's running list (2 per lane); select128() keeps the best 128 in the
+// running list in LDS.  After the last chunk each wave orders its rows' lists
+// with the bitonic network and stores them.  When the kept axis has too few
+// strips to fill the chip, the reduced axis is cut into `splits` ranges whose
+// unordered lists go to a workspace and are merged by a second kernel.
+//
+// Plays the role of topk_bmm_* with topk_dim_1 / topk_dim_2, bitonic_sort_128,
+// bitonic_sort_256 and the row mutex (reference kernels/topkbmm.cu:13-303,
+// 499-594), and of the standalone bitonic_sort kernel
+// (reference kernels/bitonic_sort.cu:182-216).
+#include "cmk_core.hpp"
+#include "cmk_launch.hpp"
+#include "cmk_select.hpp"
+
+namespace cmk {
+
+constexpr int kChunkTiles = 8;                 // tiles of 128 candidates per chunk
+constexpr int kStagePitch = 128 * kChunkTiles + 8;
+
+struct TopkArgs {
+  Operand X, Y;
+  long long strideX, strideY;
+  float* values;        // [L][Yext][k]
+  long long* indices;   // [L][Yext][k]
+  uint32_t* part_key;   // [splits][L*Yext][128]  (splits > 1)
+  int* part_idx;
+  int L, K, k;
+  int ystrips, xtiles, splits, tiles_per_split;
+};
+
+template <int XK, int YK>
+__global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
+  using C = Core<XK, YK, 4, 1, 1, 1>;
+  static_assert(C::TX == 128 && C::TY == 32, "tile shape");
+  constexpr int opFloats = C::ldsFloats;
+  static_assert(opFloats >= 8 * kStagePitch, "staging area aliases the operand buffers");
+  __shared__ __attribute__((aligned(16))) float lds[opFloats];
+  __shared__ uint32_t list_key[32][kTop];
+  __shared__ int list_idx[32][kTop];
+
+  const int total = a.L * a.ystrips * a.splits;
+  const int logical = xcd_logical_id(blockIdx.x, total);
+  if (logical < 0) return;
+  const int split = logical / (a.L * a.ystrips);
+  const int rem = logical - split * (a.L * a.ystrips);
+  const int b = rem / a.ystrips;
+  const int ystrip = rem - b * a.ystrips;
+  const int y0 = ystrip * C::TY;
+  const int xt_begin = split * a.tiles_per_split;
+  const int xt_end = min(a.xtiles, xt_begin + a.tiles_per_split);
+
+  Operand X = a.X, Y = a.Y;
+  X.p += (long long)b * a.strideX;
+  Y.p += (long long)b * a.strideY;
+  const int x_limit = min(X.rows, xt_end * C::TX);
+  const int Yext = Y.rows;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int l32 = lane & 31;
+  const int half = lane >> 5;
+
+  // running lists start empty
+  for (int e = threadIdx.x; e < 32 * kTop; e += kThreads) {
+    (&list_key[0][0])[e] = 0u;
+    (&list_idx[0][0])[e] = -1;
+  }
+  __syncthreads();
+
+  C core;
+  const int S = max(1, (a.K + KS - 1) / KS);
+
+  for (int xt0 = xt_begin; xt0 < xt_end; xt0 += kChunkTiles) {
+    const int nt = min(kChunkTiles, xt_end - xt0);
+    const int iters = nt * S;
+    __syncthreads();  // previous chunk's staging reads are finished
+    core.load(X, Y, xt0 * C::TX, y0, 0, a.K);
+    core.store(lds);
+    __syncthreads();
+    f32x16 acc[kChunkTiles][1][1];
+    int it = 0;
+#pragma unroll
+    for (int i = 0; i < kChunkTiles; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][0][0][r] = 0.f;
+      if (i < nt) {
+        for (int s = 0; s < S; ++s, ++it) {
+          const bool more = it + 1 < iters;
+          if (more) {
+            const bool wrap = (s + 1 == S);
+            core.load(X, Y, (xt0 + (wrap ? i + 1 : i)) * C::TX, y0, wrap ? 0 : (s + 1) * KS, a.K);
+          }
+          core.mma(lds + (it & 1) * C::bufFloats, acc[i]);
+          if (more) core.store(lds + ((it + 1) & 1) * C::bufFloats);
+          __syncthreads();
+        }
+      }
+    }
+
+    // selection, eight rows of the strip per pass
+    const int xc0 = xt0 * C::TX;
+#pragma unroll 1
+    for (int g = 0; g < 4; ++g) {
+      if (g) __syncthreads();  // previous pass has been read
+      if ((l32 >> 3) == g) {
+        float* row = lds + (l32 & 7) * kStagePitch + wave * 32 + 4 * half;
+#pragma unroll
+        for (int i = 0; i < kChunkTiles; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            f32x4 v = {acc[i][0][0][4 * q], acc[i][0][0][4 * q + 1], acc[i][0][0][4 * q + 2],
+                       acc[i][0][0][4 * q + 3]};
+            *reinterpret_cast<f32x4*>(row + i * 128 + 8 * q) = v;
+          }
+      }
+      __syncthreads();
+#pragma unroll 1
+      for (int rr = 0; rr < 2; ++rr) {
+        const int r = 8 * g + 2 * wave + rr;  // row of the strip, owned by this wave
+        if (y0 + r >= Yext) continue;
+        const float* src = lds + (r & 7) * kStagePitch;
+        uint32_t key[18];
+        int idx[18];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int x = xc0 + lane + 64 * j;
+          const bool ok = x < x_limit;
+          key[j] = ok ? f2key(src[lane + 64 * j]) : 0u;
+          idx[j] = ok ? x : -1;
+        }
+        key[16] = list_key[r][lane];
+        idx[16] = list_idx[r][lane];
+        key[17] = list_key[r][lane + 64];
+        idx[17] = list_idx[r][lane + 64];
+        select128<18>(key, idx, list_key[r], list_idx[r]);
+      }
+    }
+  }
+
+  // each wave finishes the rows it owns
+#pragma unroll 1
+  for (int g = 0; g < 4; ++g) {
+#pragma unroll 1
+    for (int rr = 0; rr < 2; ++rr) {
+      const int r = 8 * g + 2 * wave + rr;
+      const int y = y0 + r;
+      if (y >= Yext) continue;
+      const long long orow = (long long)b * Yext + y;
+      if (a.splits == 1) {
+        sort_and_store(list_key[r], list_idx[r], a.values + orow * a.k, a.indices + orow * a.k, a.k);
+      } else {
+        const long long o = ((long long)split * a.L * Yext + orow) * kTop;
+        a.part_key[o + lane] = list_key[r][lane];
+        a.part_idx[o + lane] = list_idx[r][lane];
+        a.part_key[o + lane + 64] = list_key[r][lane + 64];
+        a.part_idx[o + lane + 64] = list_idx[r][lane + 64];
+      }
+    }
+  }
+}
+
+// One wave per output row: folds `parts` unordered 128-entry lists into one,
+// orders it and stores the first k entries.
+__global__ __launch_bounds__(kThreads) void topk_merge_kernel(const uint32_t* part_key,
+                                                              const int* part_idx, float* values,
+                                                              long long* indices, long long rows,
+                                                              int parts, int k) {
+  __shared__ uint32_t list_key[4][kTop];
+  __shared__ int list_idx[4][kTop];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const long long row = (long long)blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  list_key[wave][lane] = 0u;
+  list_key[wave][lane + 64] = 0u;
+  list_idx[wave][lane] = -1;
+  list_idx[wave][lane + 64] = -1;
+  for (int p0 = 0; p0 < parts; p0 += 8) {
+    uint32_t key[18];
+    int idx[18];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int p = p0 + (j >> 1);
+      const bool ok = p < parts;
+      const long long o = ((long long)p * rows + row) * kTop + lane + 64 * (j & 1);
+      key[j] = ok ? part_key[o] : 0u;
+      idx[j] = ok ? part_idx[o] : -1;
+    }
+    key[16] = list_key[wave][lane];
+    idx[16] = list_idx[wave][lane];
+    key[17] = list_key[wave][lane + 64];
+    idx[17] = list_idx[wave][lane + 64];
+    select128<18>(key, idx, list_key[wave], list_idx[wave]);
+  }
+  sort_and_store(list_key[wave], list_idx[wave], values + row * k, indices + row * k, k);
+}
+
+// One wave per part of a 1-D array: keeps the best 128 of its range.
+__global__ __launch_bounds__(kThreads) void topk1d_partial_kernel(const float* arr, long long n,
+                                                                  long long span, int parts,
+                                                                  uint32_t* part_key,
+                                                                  int* part_idx) {
+  __shared__ uint32_t list_key[4][kTop];
+  __shared__ int list_idx[4][kTop];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int part = blockIdx.x * 4 + wave;
+  if (part >= parts) return;
+  list_key[wave][lane] = 0u;
+  list_key[wave][lane + 64] = 0u;
+  list_idx[wave][lane] = -1;
+  list_idx[wave][lane + 64] = -1;
+  const long long begin = (long long)part * span;
+  const long long end = begin + span < n ? begin + span : n;
+  for (long long c0 = begin; c0 < end; c0 += 1024) {
+    uint32_t key[18];
+    int idx[18];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const long long x = c0 + lane + 64 * j;
+      const bool ok = x < end;
+      key[j] = ok ? f2key(arr[x]) : 0u;
+      idx[j] = ok ? (int)x : -1;
+    }
+    key[16] = list_key[wave][lane];
+    idx[16] = list_idx[wave][lane];
+    key[17] = list_key[wave][lane + 64];
+    idx[17] = list_idx[wave][lane + 64];
+    select128<18>(key, idx, list_key[wave], list_idx[wave]);
+  }
+  const long long o = (long long)part * kTop;
+  part_key[o + lane] = list_key[wave][lane];
+  part_idx[o + lane] = list_idx[wave][lane];
+  part_key[o + lane + 64] = list_key[wave][lane + 64];
+  part_idx[o + lane + 64] = list_idx[wave][lane + 64];
+}
+
+static void plan_topk(int L, int Xext, int Yext, int* ystrips, int* xtiles, int* splits,
+                      int* tiles_per_split) {
+  *ystrips = ceil_div(Yext, 32);
+  *xtiles = ceil_div(Xext, 128);
+  const long long strips = (long long)L * *ystrips;
+  const int chunks = ceil_div(*xtiles, kChunkTiles);
+  int want = 1;
+  if (strips < 512) want = (int)((512 + strips - 1) / strips);
+  if (want > chunks) want = chunks;
+  if (want < 1) want = 1;
+  const int chunks_per_split = ceil_div(chunks, want);
+  *tiles_per_split = chunks_per_split * kChunkTiles;
+  *splits = ceil_div(*xtiles, *tiles_per_split);
+}
+
+size_t topk_workspace_bytes(int L, int Xext, int Yext) {
+  int ys, xt, sp, tps;
+  plan_topk(L, Xext, Yext, &ys, &xt, &sp, &tps);
+  if (sp <= 1) return 0;
+  return (size_t)sp * L * Yext * kTop * 8;
+}
+
+static void plan_topk1d(long long n, long long* span, int* parts) {
+  long long s = (n + 1023) / 1024;   // chunks in total
+  long long per = (s + 1023) / 1024; // chunks per part, at most 1024 parts
+  if (per < 1) per = 1;
+  *span = per * 1024;
+  *parts = (int)((n + *span - 1) / *span);
+  if (*parts < 1) *parts = 1;
+}
+
+size_t topk1d_workspace_bytes(long long n) {
+  long long span;
+  int parts;
+  plan_topk1d(n, &span, &parts);
+  return (size_t)parts * kTop * 8;
+}
+
+}  // namespace cmk
+
+using namespace cmk;
+
+extern "C" int cmk_topk_bmm_f32(const float* A, const float* B, float* values, long long* indices,
+                                const cmk_gemm_desc* d, int dim, int k, int distance,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  if (int e = check_desc(d)) return e;
+  if (dim != 1 && dim != 2) return fail(CMK_ERR_INVALID_ARG, "cmk_topk_bmm_f32: dim must be 1 or 2");
+  if (k <= 0 || k > kTop) return fail(CMK_ERR_INVALID_ARG, "cmk_topk_bmm_f32: k must be in 1..128");
+  if (distance < CMK_DIST_INNER || distance > CMK_DIST_L1)
+    return fail(CMK_ERR_INVALID_ARG, "cmk_topk_bmm_f32: unknown distance %d", distance);
+  if (distance != CMK_DIST_INNER)
+    return fail(CMK_ERR_UNSUPPORTED, "cmk_topk_bmm_f32: only distance \"inner\" is implemented");
+  const int Xext = dim == 2 ? d->N : d->M;
+  const int Yext = dim == 2 ? d->M : d->N;
+  if (d->L == 0 || Yext == 0) return CMK_OK;
+  if (!values || !indices || (d->K > 0 && Xext > 0 && (!A || !B)))
+    return fail(CMK_ERR_INVALID_ARG, "cmk_topk_bmm_f32: null pointer");
+
+  TopkArgs a{};
+  const Operand opA{A, d->lda, d->M, vec_ok(A, d->lda, d->strideA)};
+  const Operand opB{B, d->ldb, d->N, vec_ok(B, d->ldb, d->strideB)};
+  const int kindA = d->transA ? RC : KC;
+  const int kindB = d->transB ? KC : RC;
+  int xk, yk;
+  if (dim == 2) { a.X = opB; a.Y = opA; a.strideX = d->strideB; a.strideY = d->strideA; xk = kindB; yk = kindA; }
+  else          { a.X = opA; a.Y = opB; a.strideX = d->strideA; a.strideY = d->strideB; xk = kindA; yk = kindB; }
+  a.values = values;
+  a.indices = indices;
+  a.L = d->L;
+  a.K = d->K;
+  a.k = k;
+  plan_topk(d->L, Xext, Yext, &a.ystrips, &a.xtiles, &a.splits, &a.tiles_per_split);
+  if (a.xtiles == 0) { a.xtiles = 0; a.splits = 1; a.tiles_per_split = kChunkTiles; }
+  if (a.splits > 1) {
+    const size_t need = (size_t)a.splits * d->L * Yext * kTop * 8;
+    if (!workspace || workspace_bytes < need)
+      return fail(CMK_ERR_WORKSPACE, "cmk_topk_bmm_f32: workspace of %zu bytes required, %zu given",
+                  need, workspace_bytes);
+    a.part_key = static_cast<uint32_t*>(workspace);
+    a.part_idx = reinterpret_cast<int*>(a.part_key + (size_t)a.splits * d->L * Yext * kTop);
+  }
+  const long long total = (long long)d->L * a.ystrips * a.splits;
+  if (int e = check_grid(total)) return e;
+  const dim3 grid((unsigned)(((total + 7) / 8) * 8)), block(kThreads);
+  hipStream_t st = (hipStream_t)stream;
+  if (xk == KC && yk == KC) hipLaunchKernelGGL((topk_kernel<KC, KC>), grid, block, 0, st, a);
+  else if (xk == KC && yk == RC) hipLaunchKernelGGL((topk_kernel<KC, RC>), grid, block, 0, st, a);
+  else if (xk == RC && yk == KC) hipLaunchKernelGGL((topk_kernel<RC, KC>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((topk_kernel<RC, RC>), grid, block, 0, st, a);
+  if (int e = hip_status(hipGetLastError(), "cmk_topk_bmm_f32 launch")) return e;
+  if (a.splits > 1) {
+    const long long rows = (long long)d->L * Yext;
+    if (int e = check_grid((rows + 3) / 4)) return e;
+    hipLaunchKernelGGL(topk_merge_kernel, dim3((unsigned)((rows + 3) / 4)), block, 0, st,
+                       a.part_key, a.part_idx, values, indices, rows, a.splits, k);
+    if (int e = hip_status(hipGetLastError(), "cmk_topk_bmm_f32 merge launch")) return e;
+  }
+  return CMK_OK;
+}
+
+extern "C" int cmk_topk_1d_f32(const float* arr, long long n, float* values, long long* indices,
+                               int k, void* workspace, size_t workspace_bytes, void* stream) {
+  if (n < 0 || n > 0x7fffffffLL) return fail(CMK_ERR_INVALID_ARG, "cmk_topk_1d_f32: bad length");
+  if (k <= 0 || k > kTop) return fail(CMK_ERR_INVALID_ARG, "cmk_topk_1d_f32: k must be in 1..128");
+  if (!values || !indices || (n > 0 && !arr))
+    return fail(CMK_ERR_INVALID_ARG, "cmk_topk_1d_f32: null pointer");
+  long long span;
+  int parts;
+  plan_topk1d(n, &span, &parts);
+  const size_t need = (size_t)parts * kTop * 8;
+  if (!workspace || workspace_bytes < need)
+    return fail(CMK_ERR_WORKSPACE, "cmk_topk_1d_f32: workspace of %zu bytes required, %zu given",
+                need, workspace_bytes);
+  uint32_t* pk = static_cast<uint32_t*>(workspace);
+  int* pi = reinterpret_cast<int*>(pk + (size_t)parts * kTop);
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(topk1d_partial_kernel, dim3((unsigned)((parts + 3) / 4)), dim3(kThreads), 0, st,
+                     arr, n, span, parts, pk, pi);
+  if (int e = hip_status(hipGetLastError(), "cmk_topk_1d_f32 launch")) return e;
+  hipLaunchKernelGGL(topk_merge_kernel, dim3(1), dim3(kThreads), 0, st, pk, pi, values, indices,
+                     (long long)1, parts, k);
+  return hip_status(hipGetLastError(), "cmk_topk_1d_f32 merge launch");
+}

@@ -1,0 +1,53 @@
+"""Fused min / argmin of a batched fp32 product along one axis."""
+import torch
+
+from . import _common, _lib
+
+
+class MinBMMCUDA:
+    """Drop-in for the reference's ``MinBMMCUDA`` (reference minbmm.py:7-148):
+    same constructor keywords, same ``__call__(A, B, dim=1)`` returning
+    ``(values, indices)``.
+
+    `dim` is an axis of A@B as the reference counts it (for 3-D inputs 1 reduces
+    over m, 2 over n; for 2-D inputs 0 and 1); negative dims are accepted as
+    well.  Every output element is written, ties resolve to the lowest index
+    (the reference's index write is racy, kernels/minbmm.cu:76-79), and an
+    unknown `distance` raises (the reference only builds the exception,
+    minbmm.py:19).
+    """
+
+    def __init__(self, patch_m=4, patch_n=4, distance="inner"):
+        self.patch_m = patch_m
+        self.patch_n = patch_n
+        self._distance = _common.distance_code(distance)
+        self.distance = distance
+        self._lib = _lib.load()
+
+    def get_mode(self, A, B):
+        a, b = _common.get_mode(A, B)
+        return "".join([a or "n", b or "n"])
+
+    def __call__(self, A, B, dim=1):
+        A, B, two_dimensional = _common.promote(A, B)
+        dim = _common.normalize_dim(dim, two_dimensional)
+        _common.check_operands(A, B)
+        l, m, k = A.shape
+        n = B.shape[2]
+        kept, reduced = (n, m) if dim == 1 else (m, n)
+        if reduced == 0:
+            raise ValueError("min_bmm: cannot reduce over an axis of extent 0")
+        values = torch.empty([l, kept], device=A.device, dtype=A.dtype)
+        indices = torch.empty([l, kept], device=A.device, dtype=torch.int64)
+        if values.numel():
+            A2, B2, desc = _common.make_desc(A, B)
+            ws, ws_bytes = _common.workspace(_lib.OP_MIN_BMM, l, m, n, k, dim, A.device)
+            with torch.cuda.device(A.device):
+                _lib.check(self._lib.cmk_min_bmm_f32(
+                    A2.data_ptr(), B2.data_ptr(), values.data_ptr(), indices.data_ptr(), desc,
+                    dim, self._distance, ws.data_ptr() if ws is not None else None, ws_bytes,
+                    _common.stream_ptr(A.device)))
+        if two_dimensional:
+            indices = indices[0]
+            values = values[0]
+        return values, indices

@@ -1,0 +1,132 @@
+/*
+ * cmk.h - C ABI of libcmk.so, the gfx950 (MI355X) fused batched-matmul library.
+ *
+ * Every entry point enqueues work on the caller's HIP stream and returns
+ * without synchronising.  All data pointers are device pointers owned by the
+ * caller; the library never allocates or frees device memory.  Scratch space,
+ * where an operation needs it, is a caller-provided workspace whose size is
+ * reported by cmk_workspace_bytes().
+ *
+ * Matrices are fp32.  An operand is described by a pointer, a leading
+ * dimension `ld` (in elements), a batch stride (in elements) and a transpose
+ * flag:
+ *     transA == 0 : A[b][m][k] lives at  A + b*strideA + m*lda + k   ("n")
+ *     transA == 1 : A[b][m][k] lives at  A + b*strideA + k*lda + m   ("t")
+ *     transB == 0 : B[b][k][n] lives at  B + b*strideB + k*ldb + n   ("n")
+ *     transB == 1 : B[b][k][n] lives at  B + b*strideB + n*ldb + k   ("t")
+ * These are the four layouts the reference infers from tensor strides
+ * (reference bmm.py:56-66) and compiles as separate kernels
+ * (reference kernels/bmm.cu:1,93,184,276).
+ *
+ * Return value: 0 on success, otherwise a negative CMK_ERR_* code or a
+ * positive hipError_t; cmk_last_error() then holds a message for the calling
+ * thread.
+ */
+#ifndef CMK_H_
+#define CMK_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CMK_ABI_VERSION 1
+
+#define CMK_OK                 0
+#define CMK_ERR_INVALID_ARG   -1   /* bad shape / dim / k / null pointer          */
+#define CMK_ERR_UNSUPPORTED   -2   /* valid request that this build does not do   */
+#define CMK_ERR_WORKSPACE     -3   /* workspace missing or too small              */
+
+/* operation ids for cmk_workspace_bytes() */
+#define CMK_OP_BMM      0
+#define CMK_OP_MBMM     1
+#define CMK_OP_MIN_BMM  2
+#define CMK_OP_TOPK_BMM 3
+#define CMK_OP_TOPK_1D  4
+
+/* accumulate functions (reference kernels/bmm_helpers.cu:20-60) */
+#define CMK_DIST_INNER 0   /* c += a*b        ("madd")       */
+#define CMK_DIST_L2    1   /* c += (a-b)^2    ("squared_l2") */
+#define CMK_DIST_L1    2   /* c += |a-b|      ("l1")         */
+
+/* Operand description shared by all GEMM-family entry points. */
+typedef struct cmk_gemm_desc {
+  int L, M, N, K;            /* batch, rows of C, cols of C, contraction length */
+  int transA, transB;        /* 0 = "n", 1 = "t" (see above)                    */
+  long long lda, ldb;        /* leading dimensions, elements                    */
+  long long strideA, strideB;/* batch strides, elements                         */
+} cmk_gemm_desc;
+
+/*
+ * C[b][m][n] = sum_k A[b][m][k] * B[b][k][n]; C is dense row-major
+ * [L][M][N] and every element is written (no pre-zeroing needed).
+ * Replaces the launch of bmm_{nn,nt,tn,tt}
+ * (reference bmm.py:115-125, kernels/bmm.cu:184-274).
+ */
+int cmk_bmm_f32(const float* A, const float* B, float* C,
+                const cmk_gemm_desc* d, void* stream);
+
+/*
+ * Masked product: C = (A@B) * element_mask where the 128x128 tile's
+ * block_mask and the 8x8 micro-tile's thread_mask are both non-zero, else 0.
+ * Tiles whose block_mask is 0 are not computed (only zeros are written).
+ * Masks are uint8: block_mask [Lm][ceil(M/128)][ceil(N/128)], thread_mask
+ * [Lm][ceil(M/8)][ceil(N/8)], element_mask [Lm][M][N] with Lm = 1 when
+ * share_mask != 0 and Lm = L otherwise.  Only transA == transB == 0 is
+ * accepted, as in the reference.  Replaces the launch of mbmm_nn
+ * (reference mbmm.py:84-97, kernels/mbmm.cu:208-374).
+ */
+int cmk_mbmm_f32(const float* A, const float* B, float* C,
+                 const uint8_t* block_mask, const uint8_t* thread_mask,
+                 const uint8_t* element_mask, int share_mask,
+                 const cmk_gemm_desc* d, void* stream);
+
+/*
+ * Fused min/argmin of C = A@B along `dim` of C[L][M][N] (1 = over m, output
+ * [L][N]; 2 = over n, output [L][M]) without storing C.  `values` is fp32,
+ * `indices` int64; every output element is written; exact ties resolve to
+ * the lowest index.  Replaces the launch of min_bmm_{nn,nt,tn,tt}
+ * (reference minbmm.py:132-143, kernels/minbmm.cu:347-440).
+ */
+int cmk_min_bmm_f32(const float* A, const float* B,
+                    float* values, long long* indices,
+                    const cmk_gemm_desc* d, int dim, int distance,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Fused top-k (largest, sorted descending, 0 < k <= 128) of C = A@B along
+ * `dim` of C[L][M][N]: dim == 2 gives [L][M][k], dim == 1 gives [L][N][k].
+ * `values` fp32 and `indices` int64 are dense with row pitch k.  When fewer
+ * than k candidates exist the trailing slots hold -inf / -1.  Replaces the
+ * launch of topk_bmm_{nn,nt,tn,tt}
+ * (reference topkbmm.py:137-149, kernels/topkbmm.cu:499-594).
+ */
+int cmk_topk_bmm_f32(const float* A, const float* B,
+                     float* values, long long* indices,
+                     const cmk_gemm_desc* d, int dim, int k, int distance,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Top-k (largest, sorted descending, 0 < k <= 128) of a 1-D fp32 array of
+ * length n.  Replaces the launch of bitonic_sort
+ * (reference kernels/bitonic_sort.cu:182-216).
+ */
+int cmk_topk_1d_f32(const float* arr, long long n,
+                    float* values, long long* indices, int k,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* Bytes of device workspace an operation needs (0 = none).  For
+ * CMK_OP_TOPK_1D pass the array length in M (L = 1). */
+size_t cmk_workspace_bytes(int op, int L, int M, int N, int K, int dim);
+
+/* Message describing the last failure on the calling thread ("" if none). */
+const char* cmk_last_error(void);
+
+int cmk_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CMK_H_ */
