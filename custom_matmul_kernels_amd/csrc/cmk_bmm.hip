@@ -159,7 +159,7 @@ extern "C" int cmk_bmm_f32(const float* A, const float* B, float* C, const cmk_g
                            void* stream) {
   if (int e = check_desc(d)) return e;
   if (d->L == 0 || d->M == 0 || d->N == 0) return CMK_OK;
-  if (!A || !B || !C) return fail(CMK_ERR_INVALID_ARG, "cmk_bmm_f32: null pointer");
+  if (!C || (d->K > 0 && (!A || !B))) return fail(CMK_ERR_INVALID_ARG, "cmk_bmm_f32: null pointer");
   if (int e = check_grid((long long)d->L * ((d->M + 127) / 128) * ((d->N + 127) / 128))) return e;
   BmmArgs a = make_args(A, B, C, d);
   return hip_status(launch_bmm<false>(a, d->transA, d->transB, (hipStream_t)stream),
@@ -173,7 +173,7 @@ extern "C" int cmk_mbmm_f32(const float* A, const float* B, float* C, const uint
   if (d->transA || d->transB)
     return fail(CMK_ERR_UNSUPPORTED, "cmk_mbmm_f32: only the \"nn\" layout is implemented");
   if (d->L == 0 || d->M == 0 || d->N == 0) return CMK_OK;
-  if (!A || !B || !C || !block_mask || !thread_mask || !element_mask)
+  if (!C || (d->K > 0 && (!A || !B)) || !block_mask || !thread_mask || !element_mask)
     return fail(CMK_ERR_INVALID_ARG, "cmk_mbmm_f32: null pointer");
   if (int e = check_grid((long long)d->L * ((d->M + 127) / 128) * ((d->N + 127) / 128))) return e;
   BmmArgs a = make_args(A, B, C, d);
