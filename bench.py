@@ -91,6 +91,17 @@ def make_workloads(torch, cmk, dev):
                        desc="mbmm fp32 A[%d,%d,%d] @ B[%d,%d,%d], tril & tile-Bernoulli(0.5) mask" % (L, M, K, L, K, N),
                        bytes=4.0 * L * (M * N + M * K + K * N) + L * M * N + L * (M // 8) * (N // 8))
 
+    def copy_wl(name, nbytes):
+        # a plain device copy of known size: the yardstick the HBM counters are scaled by
+        def make():
+            src = torch.empty(nbytes // 4, dtype=torch.float32, device=dev).normal_()
+            return src, torch.empty_like(src)
+
+        W[name] = dict(make=make, run=lambda src, dst: dst.copy_(src), flop=0.0,
+                       desc="device copy of %d bytes (reads and writes that many)" % nbytes,
+                       bytes=2.0 * nbytes)
+
+    copy_wl("copy_probe", 1 << 30)
     min_wl("min_bmm_large", 65536, 65536, 256, cpu_rows=4096)
     min_wl("min_bmm_small", 4096, 4096, 64, cpu_rows=4096)
     topk_wl("topk_bmm", 1048576, 1024, 256, cpu_rows=65536)
@@ -124,12 +135,13 @@ def cpu_baseline(torch, wl, args_dev, budget_s=12.0):
     if "cpu" not in wl:
         return None
     A, B = args_dev[0].cpu(), args_dev[1].cpu()
-    torch.set_num_threads(os.cpu_count() or 1)
     wl["cpu"](A, B)                                  # warm-up slab
     done_rows, t_total = 0, 0.0
     rows = wl["cpu_rows"]
     off = 0
-    while t_total < budget_s and off + rows <= wl["rows"] and done_rows < 4 * rows:
+    while t_total < budget_s and done_rows < 8 * wl["rows"]:
+        if off + rows > wl["rows"]:
+            off = 0                                  # another pass over the same rows
         a = A[:, off:off + rows]
         t0 = time.perf_counter()
         wl["cpu"](a, B)
@@ -196,7 +208,7 @@ def main():
     if not a.no_others:
         others = {}
         for name, w in W.items():
-            if name == a.workload:
+            if name == a.workload or name == "copy_probe":
                 continue
             steps = 5 if name == "topk_bmm" else 20
             args, ms_o, kern_o = run_workload(torch, w, steps, 3)

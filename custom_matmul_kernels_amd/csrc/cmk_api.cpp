@@ -47,19 +47,18 @@ int check_grid(long long work_groups) {
   return CMK_OK;
 }
 
-size_t min_workspace_bytes(int L, int Xext, int Yext);
+size_t min_workspace_bytes(int L, int Xext, int Yext, int K);
 size_t topk_workspace_bytes(int L, int Xext, int Yext);
 size_t topk1d_workspace_bytes(long long n);
 
 }  // namespace cmk
 
 extern "C" size_t cmk_workspace_bytes(int op, int L, int M, int N, int K, int dim) {
-  (void)K;
   if (L < 0 || M < 0 || N < 0) return 0;
   switch (op) {
     case CMK_OP_MIN_BMM:
       if (dim != 1 && dim != 2) return 0;
-      return cmk::min_workspace_bytes(L, dim == 2 ? N : M, dim == 2 ? M : N);
+      return cmk::min_workspace_bytes(L, dim == 2 ? N : M, dim == 2 ? M : N, K);
     case CMK_OP_TOPK_BMM:
       if (dim != 1 && dim != 2) return 0;
       return cmk::topk_workspace_bytes(L, dim == 2 ? N : M, dim == 2 ? M : N);

@@ -9,7 +9,7 @@
 // axis in X (running state stays in one lane), a row-major store wants the
 // contiguous axis in Y (a store instruction writes 128-byte row segments).
 //
-// The contraction is walked in slabs of KS = 32.  A slab of each operand is
+// The contraction is walked in slabs of KS (32 unless a kernel asks otherwise).  A slab of each operand is
 // fetched from global memory into registers, written to one of two LDS
 // buffers, and consumed from the other with v_mfma_f32_32x32x2_f32.  Inside a
 // slab, k is consumed in groups of 8: lanes 0-31 feed k = 8g+0..3 and lanes
@@ -35,7 +35,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
-constexpr int KS = 32;  // contraction depth of one LDS slab
 constexpr int KC = 0;   // k-contiguous operand
 constexpr int RC = 1;   // row-contiguous operand
 
@@ -46,92 +45,108 @@ struct Operand {
   int vec;         // non-zero when 16-byte loads are legal (base and ld aligned)
 };
 
-template <int KIND, int T>
+// LDS footprint of one slab (KS deep) of a T-row operand tile.
+template <int KIND, int T, int KS>
 struct TileLayout;
-template <int T>
-struct TileLayout<KC, T> {
+template <int T, int KS>
+struct TileLayout<KC, T, KS> {
   static constexpr int pitch = KS + 4;
   static constexpr int floats = T * pitch;
 };
-template <int T>
-struct TileLayout<RC, T> {
+template <int T, int KS>
+struct TileLayout<RC, T, KS> {
   static constexpr int pitch = T + 8;
   static constexpr int floats = KS * pitch;
 };
 
 // ---- global -> registers ---------------------------------------------------
-template <int KIND, int T>
+// Each thread fetches NV = T*KS/1024 groups of four consecutive floats.  A tile
+// that lies completely inside the matrix takes the branch-free path.
+template <int KIND, int T, int KS>
 __device__ __forceinline__ void gload(const Operand& o, int r0, int k0, int K,
-                                      f32x4 (&v)[T / 32]) {
+                                      f32x4 (&v)[T * KS / 1024]) {
+  constexpr int NV = T * KS / 1024;
   const int t = threadIdx.x;
+  const bool interior = o.vec && (k0 + KS <= K) && (r0 + T <= o.rows);  // uniform
   if constexpr (KIND == KC) {
-    const int kk = k0 + (t & 7) * 4;
-    const int rr = r0 + (t >> 3);
+    constexpr int TPR = KS / 4;          // threads per row
+    constexpr int RPP = kThreads / TPR;  // rows per pass
+    const int kk = k0 + (t % TPR) * 4;
+    const int rr = r0 + t / TPR;
+    if (interior) {
+      const float* src = o.p + (long long)rr * o.ld + kk;
 #pragma unroll
-    for (int p = 0; p < T / 32; ++p) {
-      const int row = rr + 32 * p;
-      f32x4 val = {0.f, 0.f, 0.f, 0.f};
-      if (row < o.rows) {
+      for (int p = 0; p < NV; ++p)
+        v[p] = *reinterpret_cast<const f32x4*>(src + (long long)p * RPP * o.ld);
+    } else if (K > 0 && o.rows > 0) {
+      // edge tile: every element is fetched from a clamped (always valid)
+      // address and zeroed when it lies outside the matrix; no divergent branches
+#pragma unroll
+      for (int p = 0; p < NV; ++p) {
+        const int row = rr + RPP * p;
         const float* src = o.p + (long long)row * o.ld + kk;
-        if (o.vec && kk + 3 < K) {
-          val = *reinterpret_cast<const f32x4*>(src);
-        } else {
-          if (kk + 0 < K) val.x = src[0];
-          if (kk + 1 < K) val.y = src[1];
-          if (kk + 2 < K) val.z = src[2];
-          if (kk + 3 < K) val.w = src[3];
-        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[p][j] = *((row < o.rows && kk + j < K) ? src + j : o.p);
       }
-      v[p] = val;
+#pragma unroll
+      for (int p = 0; p < NV; ++p) {
+        const int row = rr + RPP * p;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[p][j] = (row < o.rows && kk + j < K) ? v[p][j] : 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < NV; ++p) v[p] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
   } else {
     constexpr int TPR = T / 4;           // threads per k-row
     constexpr int RPP = kThreads / TPR;  // k-rows per pass
     const int rr = r0 + (t % TPR) * 4;
     const int kb = k0 + t / TPR;
+    if (interior) {
+      const float* src = o.p + (long long)kb * o.ld + rr;
 #pragma unroll
-    for (int p = 0; p < T / 32; ++p) {
-      const int kk = kb + p * RPP;
-      f32x4 val = {0.f, 0.f, 0.f, 0.f};
-      if (kk < K) {
+      for (int p = 0; p < NV; ++p)
+        v[p] = *reinterpret_cast<const f32x4*>(src + (long long)p * RPP * o.ld);
+    } else if (K > 0 && o.rows > 0) {
+#pragma unroll
+      for (int p = 0; p < NV; ++p) {
+        const int kk = kb + p * RPP;
         const float* src = o.p + (long long)kk * o.ld + rr;
-        if (o.vec && rr + 3 < o.rows) {
-          val = *reinterpret_cast<const f32x4*>(src);
-        } else {
-          if (rr + 0 < o.rows) val.x = src[0];
-          if (rr + 1 < o.rows) val.y = src[1];
-          if (rr + 2 < o.rows) val.z = src[2];
-          if (rr + 3 < o.rows) val.w = src[3];
-        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[p][j] = *((kk < K && rr + j < o.rows) ? src + j : o.p);
       }
-      v[p] = val;
+#pragma unroll
+      for (int p = 0; p < NV; ++p) {
+        const int kk = kb + p * RPP;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[p][j] = (kk < K && rr + j < o.rows) ? v[p][j] : 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < NV; ++p) v[p] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
   }
 }
 
 // ---- registers -> LDS --------------------------------------------------------
-template <int KIND, int T>
-__device__ __forceinline__ void lstore(float* lds, const f32x4 (&v)[T / 32]) {
+template <int KIND, int T, int KS>
+__device__ __forceinline__ void lstore(float* lds, const f32x4 (&v)[T * KS / 1024]) {
+  constexpr int NV = T * KS / 1024;
   const int t = threadIdx.x;
-  constexpr int pitch = TileLayout<KIND, T>::pitch;
-  if constexpr (KIND == KC) {
+  constexpr int pitch = TileLayout<KIND, T, KS>::pitch;
+  constexpr int TPR = KIND == KC ? KS / 4 : T / 4;
+  constexpr int RPP = kThreads / TPR;
 #pragma unroll
-    for (int p = 0; p < T / 32; ++p)
-      *reinterpret_cast<f32x4*>(&lds[((t >> 3) + 32 * p) * pitch + (t & 7) * 4]) = v[p];
-  } else {
-    constexpr int TPR = T / 4;
-    constexpr int RPP = kThreads / TPR;
-#pragma unroll
-    for (int p = 0; p < T / 32; ++p)
-      *reinterpret_cast<f32x4*>(&lds[(t / TPR + p * RPP) * pitch + (t % TPR) * 4]) = v[p];
-  }
+  for (int p = 0; p < NV; ++p)
+    *reinterpret_cast<f32x4*>(&lds[(t / TPR + p * RPP) * pitch + (t % TPR) * 4]) = v[p];
 }
 
 // ---- LDS -> MFMA fragment ----------------------------------------------------
 // Four k values (8*kg + 4*half + 0..3) of tile row `row` for this lane.
-template <int KIND, int T>
+template <int KIND, int T, int KS>
 __device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg, int half) {
-  constexpr int pitch = TileLayout<KIND, T>::pitch;
+  constexpr int pitch = TileLayout<KIND, T, KS>::pitch;
   if constexpr (KIND == KC) {
     return *reinterpret_cast<const f32x4*>(&lds[row * pitch + kg * 8 + half * 4]);
   } else {
@@ -146,30 +161,34 @@ __device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg, int hal
 }
 
 // Work-group level tile engine.  WX x WY waves (WX*WY == 4), each wave owns
-// BX x BY blocks of 32x32.
-template <int XK, int YK, int WX, int WY, int BX, int BY>
+// BX x BY blocks of 32x32; KS is the contraction depth of one LDS slab.
+template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32>
 struct Core {
   static_assert(WX * WY == 4, "four waves per work-group");
+  static constexpr int KS = KS_;
   static constexpr int TX = WX * BX * 32;
   static constexpr int TY = WY * BY * 32;
-  static constexpr int xFloats = TileLayout<XK, TX>::floats;
-  static constexpr int yFloats = TileLayout<YK, TY>::floats;
+  static_assert(KS % 8 == 0 && (TX * KS) % 1024 == 0 && (TY * KS) % 1024 == 0, "tile shape");
+  static constexpr int xFloats = TileLayout<XK, TX, KS>::floats;
+  static constexpr int yFloats = TileLayout<YK, TY, KS>::floats;
   static constexpr int bufFloats = xFloats + yFloats;
   static constexpr int ldsFloats = 2 * bufFloats;
 
-  f32x4 xv[TX / 32];
-  f32x4 yv[TY / 32];
+  f32x4 xv[TX * KS / 1024];
+  f32x4 yv[TY * KS / 1024];
 
   __device__ __forceinline__ void load(const Operand& X, const Operand& Y, int x0, int y0,
                                        int k0, int K) {
-    gload<XK, TX>(X, x0, k0, K, xv);
-    gload<YK, TY>(Y, y0, k0, K, yv);
+    gload<XK, TX, KS>(X, x0, k0, K, xv);
+    gload<YK, TY, KS>(Y, y0, k0, K, yv);
   }
   __device__ __forceinline__ void store(float* buf) {
-    lstore<XK, TX>(buf, xv);
-    lstore<YK, TY>(buf + xFloats, yv);
+    lstore<XK, TX, KS>(buf, xv);
+    lstore<YK, TY, KS>(buf + xFloats, yv);
   }
-  // acc[bx][by] += X-block(bx) * Y-block(by) over the slab held in `buf`.
+  // acc[bx][by] += X-block(bx) * Y-block(by) over the slab held in `buf`.  The
+  // fragments of k-group g+1 are fetched from LDS before the MFMAs of group g
+  // are issued, so the matrix pipe does not wait for LDS.
   __device__ __forceinline__ void mma(const float* buf, f32x16 (&acc)[BX][BY]) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -179,21 +198,31 @@ struct Core {
     const int yr = (wave / WX) * BY * 32 + l32;
     const float* bx_ = buf;
     const float* by_ = buf + xFloats;
+    constexpr int NG = KS / 8;
+    f32x4 xf[2][BX], yf[2][BY];
 #pragma unroll
-    for (int kg = 0; kg < KS / 8; ++kg) {
-      f32x4 xf[BX], yf[BY];
+    for (int b = 0; b < BX; ++b) xf[0][b] = frag<XK, TX, KS>(bx_, xr + 32 * b, 0, half);
 #pragma unroll
-      for (int b = 0; b < BX; ++b) xf[b] = frag<XK, TX>(bx_, xr + 32 * b, kg, half);
+    for (int b = 0; b < BY; ++b) yf[0][b] = frag<YK, TY, KS>(by_, yr + 32 * b, 0, half);
 #pragma unroll
-      for (int b = 0; b < BY; ++b) yf[b] = frag<YK, TY>(by_, yr + 32 * b, kg, half);
+    for (int kg = 0; kg < NG; ++kg) {
+      const int cur = kg & 1, nxt = cur ^ 1;
+      if (kg + 1 < NG) {
+#pragma unroll
+        for (int b = 0; b < BX; ++b) xf[nxt][b] = frag<XK, TX, KS>(bx_, xr + 32 * b, kg + 1, half);
+#pragma unroll
+        for (int b = 0; b < BY; ++b) yf[nxt][b] = frag<YK, TY, KS>(by_, yr + 32 * b, kg + 1, half);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the LDS reads above the MFMAs they overlap with
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int bx = 0; bx < BX; ++bx)
 #pragma unroll
           for (int by = 0; by < BY; ++by)
-            acc[bx][by] =
-                __builtin_amdgcn_mfma_f32_32x32x2f32(xf[bx][j], yf[by][j], acc[bx][by], 0, 0, 0);
+            acc[bx][by] = __builtin_amdgcn_mfma_f32_32x32x2f32(xf[cur][bx][j], yf[cur][by][j],
+                                                               acc[bx][by], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 };

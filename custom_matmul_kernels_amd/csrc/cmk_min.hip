@@ -28,6 +28,8 @@ struct MinArgs {
   int* part_idx;
   int L, K;
   int ystrips, xtiles, splits, tiles_per_split;
+  int ygroup;                   // y strips that run side by side with all their splits
+  int total;                    // work-groups with real work slots (before XCD padding)
 };
 
 template <int XK, int YK>
@@ -35,15 +37,20 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
   using C = Core<XK, YK, 2, 2, 2, 2>;
   __shared__ __attribute__((aligned(16))) float lds[C::ldsFloats];
 
-  const int total = a.L * a.ystrips * a.splits;
-  const int logical = xcd_logical_id(blockIdx.x, total);
+  // Work-groups that are resident on one XCD at the same time form a block of
+  // `ygroup` y strips x `splits` ranges of X: the strips of Y they re-read for
+  // every tile stay in that XCD's L2, and each X tile is fetched once for the
+  // `ygroup` work-groups that walk the same range.
+  const int logical = xcd_logical_id(blockIdx.x, a.total);
   if (logical < 0) return;
-  // split is the slowest index: work-groups that run together walk the same
-  // range of X and share its tiles in L2
-  const int split = logical / (a.L * a.ystrips);
-  const int rem = logical - split * (a.L * a.ystrips);
-  const int b = rem / a.ystrips;
-  const int ystrip = rem - b * a.ystrips;
+  const int gsz = a.ygroup * a.splits;
+  const int group = logical / gsz;
+  const int within = logical - group * gsz;
+  const int split = within / a.ygroup;
+  const int yflat = group * a.ygroup + within % a.ygroup;
+  if (yflat >= a.L * a.ystrips) return;
+  const int b = yflat / a.ystrips;
+  const int ystrip = yflat - b * a.ystrips;
   const int y0 = ystrip * C::TY;
   const int xt_begin = split * a.tiles_per_split;
   const int xt_end = min(a.xtiles, xt_begin + a.tiles_per_split);
@@ -62,7 +69,7 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
   int bidx[2] = {xt_begin * C::TX, xt_begin * C::TX};
 
   C core;
-  const int S = max(1, (a.K + KS - 1) / KS);
+  const int S = max(1, (a.K + C::KS - 1) / C::KS);
   const int iters = (xt_end - xt_begin) * S;
   if (iters > 0) {
     core.load(X, Y, xt_begin * C::TX, y0, 0, a.K);
@@ -82,7 +89,7 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
       const bool more = it + 1 < iters;
       if (more) {
         const bool wrap = (s + 1 == S);
-        core.load(X, Y, (wrap ? xt + 1 : xt) * C::TX, y0, wrap ? 0 : (s + 1) * KS, a.K);
+        core.load(X, Y, (wrap ? xt + 1 : xt) * C::TX, y0, wrap ? 0 : (s + 1) * C::KS, a.K);
       }
       core.mma(lds + (it & 1) * C::bufFloats, acc);
       if (s == S - 1) {
@@ -178,24 +185,28 @@ __global__ void min_fold_kernel(const float* part_val, const int* part_idx, floa
   indices[i] = idx;
 }
 
-// How the reduced axis is cut: enough work-groups to give every CU a couple,
-// never more splits than tiles.
-static void plan_min(int L, int Xext, int Yext, int* ystrips, int* xtiles, int* splits,
-                     int* tiles_per_split) {
+// How the work is cut.  The reduced axis is split (a) when the kept axis alone
+// does not give every CU a couple of work-groups and (b) when X is too large
+// to stay in an XCD's L2, so that fewer distinct Y strips are live per XCD.
+static void plan_min(int L, int Xext, int Yext, int K, int* ystrips, int* xtiles, int* splits,
+                     int* tiles_per_split, int* ygroup) {
   *ystrips = ceil_div(Yext, 128);
   *xtiles = ceil_div(Xext, 128);
   const long long strips = (long long)L * *ystrips;
   int want = 1;
   if (strips < 512) want = (int)((512 + strips - 1) / strips);
+  if ((long long)Xext * K * 4 > (2ll << 20) && *xtiles >= 32 && want < 4) want = 4;
   if (want > *xtiles) want = *xtiles;
+  if (want > 64) want = 64;
   if (want < 1) want = 1;
   *tiles_per_split = ceil_div(*xtiles, want);
   *splits = ceil_div(*xtiles, *tiles_per_split);
+  *ygroup = 64 / *splits > 0 ? 64 / *splits : 1;
 }
 
-size_t min_workspace_bytes(int L, int Xext, int Yext) {
-  int ys, xt, sp, tps;
-  plan_min(L, Xext, Yext, &ys, &xt, &sp, &tps);
+size_t min_workspace_bytes(int L, int Xext, int Yext, int K) {
+  int ys, xt, sp, tps, yg;
+  plan_min(L, Xext, Yext, K, &ys, &xt, &sp, &tps, &yg);
   if (sp <= 1) return 0;
   return (size_t)sp * L * Yext * 8;
 }
@@ -234,7 +245,7 @@ extern "C" int cmk_min_bmm_f32(const float* A, const float* B, float* values, lo
   a.indices = indices;
   a.L = d->L;
   a.K = d->K;
-  plan_min(d->L, Xext, Yext, &a.ystrips, &a.xtiles, &a.splits, &a.tiles_per_split);
+  plan_min(d->L, Xext, Yext, d->K, &a.ystrips, &a.xtiles, &a.splits, &a.tiles_per_split, &a.ygroup);
   if (a.splits > 1) {
     const size_t need = (size_t)a.splits * d->L * Yext * 8;
     if (!workspace || workspace_bytes < need)
@@ -243,8 +254,10 @@ extern "C" int cmk_min_bmm_f32(const float* A, const float* B, float* values, lo
     a.part_val = static_cast<float*>(workspace);
     a.part_idx = reinterpret_cast<int*>(a.part_val + (size_t)a.splits * d->L * Yext);
   }
-  const long long total = (long long)d->L * a.ystrips * a.splits;
+  const long long ytot = (long long)d->L * a.ystrips;
+  const long long total = ((ytot + a.ygroup - 1) / a.ygroup) * a.ygroup * a.splits;
   if (int e = check_grid(total)) return e;
+  a.total = (int)total;
   const dim3 grid((unsigned)(((total + 7) / 8) * 8)), block(kThreads);
   hipStream_t st = (hipStream_t)stream;
   if (xk == KC && yk == KC) hipLaunchKernelGGL((min_kernel<KC, KC>), grid, block, 0, st, a);

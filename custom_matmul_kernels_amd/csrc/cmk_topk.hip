@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
   __syncthreads();
 
   C core;
-  const int S = max(1, (a.K + KS - 1) / KS);
+  const int S = max(1, (a.K + C::KS - 1) / C::KS);
 
   for (int xt0 = xt_begin; xt0 < xt_end; xt0 += kChunkTiles) {
     const int nt = min(kChunkTiles, xt_end - xt0);
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
           const bool more = it + 1 < iters;
           if (more) {
             const bool wrap = (s + 1 == S);
-            core.load(X, Y, (xt0 + (wrap ? i + 1 : i)) * C::TX, y0, wrap ? 0 : (s + 1) * KS, a.K);
+            core.load(X, Y, (xt0 + (wrap ? i + 1 : i)) * C::TX, y0, wrap ? 0 : (s + 1) * C::KS, a.K);
           }
           core.mma(lds + (it & 1) * C::bufFloats, acc[i]);
           if (more) core.store(lds + ((it + 1) & 1) * C::bufFloats);

@@ -46,9 +46,12 @@ def test_desc_layout_matches_header():
 
 
 def test_workspace_sizes(lib):
-    # full-height strips already fill the chip: no split, no workspace
-    assert lib.cmk_workspace_bytes(_lib.OP_MIN_BMM, 1, 65536, 65536, 256, 2) == 0
+    # a small reduced operand with many strips: no split, no workspace
+    assert lib.cmk_workspace_bytes(_lib.OP_MIN_BMM, 1, 65536, 1024, 256, 2) == 0
     assert lib.cmk_workspace_bytes(_lib.OP_TOPK_BMM, 1, 1048576, 1024, 256, 2) == 0
+    # a large reduced operand is cut in a few ranges for L2 locality: 8 bytes per row and range
+    w = lib.cmk_workspace_bytes(_lib.OP_MIN_BMM, 1, 65536, 65536, 256, 2)
+    assert 0 < w <= 16 * 65536 * 8 and w % (65536 * 8) == 0
     assert lib.cmk_workspace_bytes(_lib.OP_BMM, 128, 1024, 1024, 128, 0) == 0
     # few strips: the reduced axis is split and partials need room
     w = lib.cmk_workspace_bytes(_lib.OP_MIN_BMM, 1, 4096, 4096, 64, 2)
