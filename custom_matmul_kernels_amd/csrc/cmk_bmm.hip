@@ -86,17 +86,8 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int S = max(1, (a.K + C::KS - 1) / C::KS);
-  core.load(X, Y, m0, n0, 0, a.K);
-  core.store(lds);
-  __syncthreads();
-  for (int s = 0; s < S; ++s) {
-    const bool more = s + 1 < S;
-    if (more) core.load(X, Y, m0, n0, (s + 1) * C::KS, a.K);
-    core.mma(lds + (s & 1) * C::bufFloats, acc);
-    if (more) core.store(lds + ((s + 1) & 1) * C::bufFloats);
-    __syncthreads();
-  }
+  core.begin(X, Y, m0, n0, a.K, 1, lds);
+  core.tile(X, Y, lds, acc);
 
   // epilogue
   const int mw = m0 + (wave % 2) * 64;

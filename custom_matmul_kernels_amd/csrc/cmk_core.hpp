@@ -162,67 +162,111 @@ __device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg, int hal
 
 // Work-group level tile engine.  WX x WY waves (WX*WY == 4), each wave owns
 // BX x BY blocks of 32x32; KS is the contraction depth of one LDS slab.
+//
+// The engine walks a flat sequence of slabs: `ntiles` consecutive X tiles
+// (starting at element `xbase`) against one Y strip, S = ceil(K/KS) slabs per
+// tile.  While slab i is multiplied, slab i+1 is written to the other LDS
+// buffer (in the middle of the slab, so the writes hide behind MFMAs) and slab
+// i+2 is on its way from global memory.  The one barrier per slab sits before
+// the last k-group; right after it the first fragments of slab i+1 are read,
+// so the matrix pipe keeps running across slab and tile boundaries.
 template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32>
 struct Core {
   static_assert(WX * WY == 4, "four waves per work-group");
   static constexpr int KS = KS_;
+  static constexpr int NG = KS / 8;            // k-groups per slab
+  static constexpr int WRITE_AT = NG / 2 - 1;  // k-group after which the next slab goes to LDS
   static constexpr int TX = WX * BX * 32;
   static constexpr int TY = WY * BY * 32;
-  static_assert(KS % 8 == 0 && (TX * KS) % 1024 == 0 && (TY * KS) % 1024 == 0, "tile shape");
+  static_assert(NG >= 2 && NG % 2 == 0 && (TX * KS) % 1024 == 0 && (TY * KS) % 1024 == 0,
+                "tile shape");
   static constexpr int xFloats = TileLayout<XK, TX, KS>::floats;
   static constexpr int yFloats = TileLayout<YK, TY, KS>::floats;
   static constexpr int bufFloats = xFloats + yFloats;
   static constexpr int ldsFloats = 2 * bufFloats;
 
-  f32x4 xv[TX * KS / 1024];
+  f32x4 xv[TX * KS / 1024];  // slab in flight from global memory
   f32x4 yv[TY * KS / 1024];
+  f32x4 xf[2][BX];           // fragments; [0] holds k-group 0 of the current slab at slab entry
+  f32x4 yf[2][BY];
+  int it, iters, S;          // flat slab counter
+  int lt, ls;                // (tile, slab) of the next slab to fetch
+  int xbase, y0, K;
+  int xr, yr, half;
 
-  __device__ __forceinline__ void load(const Operand& X, const Operand& Y, int x0, int y0,
-                                       int k0, int K) {
-    gload<XK, TX, KS>(X, x0, k0, K, xv);
-    gload<YK, TY, KS>(Y, y0, k0, K, yv);
+  __device__ __forceinline__ void load(const Operand& X, const Operand& Y) {
+    gload<XK, TX, KS>(X, xbase + lt * TX, ls * KS, K, xv);
+    gload<YK, TY, KS>(Y, y0, ls * KS, K, yv);
+    if (++ls == S) { ls = 0; ++lt; }
   }
   __device__ __forceinline__ void store(float* buf) {
     lstore<XK, TX, KS>(buf, xv);
     lstore<YK, TY, KS>(buf + xFloats, yv);
   }
-  // acc[bx][by] += X-block(bx) * Y-block(by) over the slab held in `buf`.  The
-  // fragments of k-group g+1 are fetched from LDS before the MFMAs of group g
-  // are issued, so the matrix pipe does not wait for LDS.
-  __device__ __forceinline__ void mma(const float* buf, f32x16 (&acc)[BX][BY]) {
+  __device__ __forceinline__ void read_frags(const float* buf, int kg, f32x4 (&fx)[BX],
+                                             f32x4 (&fy)[BY]) {
+#pragma unroll
+    for (int b = 0; b < BX; ++b) fx[b] = frag<XK, TX, KS>(buf, xr + 32 * b, kg, half);
+#pragma unroll
+    for (int b = 0; b < BY; ++b) fy[b] = frag<YK, TY, KS>(buf + xFloats, yr + 32 * b, kg, half);
+  }
+
+  // Fills the pipeline: slab 0 in LDS with its first fragments in registers,
+  // slab 1 in flight.  Ends with every wave past a barrier.
+  __device__ __forceinline__ void begin(const Operand& X, const Operand& Y, int xbase_, int y0_,
+                                        int K_, int ntiles, float* lds) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int l32 = lane & 31;
-    const int half = lane >> 5;
-    const int xr = (wave % WX) * BX * 32 + l32;
-    const int yr = (wave / WX) * BY * 32 + l32;
-    const float* bx_ = buf;
-    const float* by_ = buf + xFloats;
-    constexpr int NG = KS / 8;
-    f32x4 xf[2][BX], yf[2][BY];
+    half = lane >> 5;
+    xr = (wave % WX) * BX * 32 + (lane & 31);
+    yr = (wave / WX) * BY * 32 + (lane & 31);
+    xbase = xbase_;
+    y0 = y0_;
+    K = K_;
+    S = max(1, (K + KS - 1) / KS);
+    iters = ntiles * S;
+    it = 0;
+    lt = 0;
+    ls = 0;
+    load(X, Y);
+    store(lds);
+    __syncthreads();
+    read_frags(lds, 0, xf[0], yf[0]);
+    if (iters > 1) load(X, Y);
+  }
+
+  // acc += the current tile's product: S slabs of the flat sequence.
+  __device__ __forceinline__ void tile(const Operand& X, const Operand& Y, float* lds,
+                                       f32x16 (&acc)[BX][BY]) {
+    for (int s = 0; s < S; ++s) {
+      const float* cur = lds + (it & 1) * bufFloats;
+      float* nxt = lds + ((it + 1) & 1) * bufFloats;
+      const bool has1 = it + 1 < iters;
+      const bool has2 = it + 2 < iters;
 #pragma unroll
-    for (int b = 0; b < BX; ++b) xf[0][b] = frag<XK, TX, KS>(bx_, xr + 32 * b, 0, half);
+      for (int kg = 0; kg < NG; ++kg) {
+        if (kg + 1 < NG) {
+          read_frags(cur, kg + 1, xf[(kg + 1) & 1], yf[(kg + 1) & 1]);
+        } else if (has1) {
+          __syncthreads();
+          read_frags(nxt, 0, xf[0], yf[0]);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // LDS reads stay above the MFMAs they overlap with
 #pragma unroll
-    for (int b = 0; b < BY; ++b) yf[0][b] = frag<YK, TY, KS>(by_, yr + 32 * b, 0, half);
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-    for (int kg = 0; kg < NG; ++kg) {
-      const int cur = kg & 1, nxt = cur ^ 1;
-      if (kg + 1 < NG) {
+          for (int bx = 0; bx < BX; ++bx)
 #pragma unroll
-        for (int b = 0; b < BX; ++b) xf[nxt][b] = frag<XK, TX, KS>(bx_, xr + 32 * b, kg + 1, half);
-#pragma unroll
-        for (int b = 0; b < BY; ++b) yf[nxt][b] = frag<YK, TY, KS>(by_, yr + 32 * b, kg + 1, half);
+            for (int by = 0; by < BY; ++by)
+              acc[bx][by] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                  xf[kg & 1][bx][j], yf[kg & 1][by][j], acc[bx][by], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kg == WRITE_AT) {
+          if (has1) store(nxt);
+          if (has2) load(X, Y);
+        }
       }
-      __builtin_amdgcn_sched_barrier(0);  // keep the LDS reads above the MFMAs they overlap with
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int bx = 0; bx < BX; ++bx)
-#pragma unroll
-          for (int by = 0; by < BY; ++by)
-            acc[bx][by] = __builtin_amdgcn_mfma_f32_32x32x2f32(xf[cur][bx][j], yf[cur][by][j],
-                                                               acc[bx][by], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
+      ++it;
     }
   }
 };

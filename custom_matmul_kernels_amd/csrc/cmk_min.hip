@@ -69,14 +69,7 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
   int bidx[2] = {xt_begin * C::TX, xt_begin * C::TX};
 
   C core;
-  const int S = max(1, (a.K + C::KS - 1) / C::KS);
-  const int iters = (xt_end - xt_begin) * S;
-  if (iters > 0) {
-    core.load(X, Y, xt_begin * C::TX, y0, 0, a.K);
-    core.store(lds);
-  }
-  __syncthreads();
-  int it = 0;
+  core.begin(X, Y, xt_begin * C::TX, y0, a.K, xt_end - xt_begin, lds);
   for (int xt = xt_begin; xt < xt_end; ++xt) {
     f32x16 acc[2][2];
 #pragma unroll
@@ -85,47 +78,37 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    for (int s = 0; s < S; ++s, ++it) {
-      const bool more = it + 1 < iters;
-      if (more) {
-        const bool wrap = (s + 1 == S);
-        core.load(X, Y, (wrap ? xt + 1 : xt) * C::TX, y0, wrap ? 0 : (s + 1) * C::KS, a.K);
-      }
-      core.mma(lds + (it & 1) * C::bufFloats, acc);
-      if (s == S - 1) {
-        // fold this tile into the running minimum; indices ascend within a
-        // lane, so a strict '<' keeps the first occurrence
-        const int xb = xt * C::TX + wx * 64;
-        if (xb + 64 <= X.rows) {
+    core.tile(X, Y, lds, acc);
+    // fold this tile into the running minimum; indices ascend within a lane,
+    // so a strict '<' keeps the first occurrence
+    const int xb = xt * C::TX + wx * 64;
+    if (xb + 64 <= X.rows) {
 #pragma unroll
-          for (int bx = 0; bx < 2; ++bx)
+      for (int bx = 0; bx < 2; ++bx)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int x = xb + bx * 32 + acc_row(r, half);
+        for (int r = 0; r < 16; ++r) {
+          const int x = xb + bx * 32 + acc_row(r, half);
 #pragma unroll
-              for (int by = 0; by < 2; ++by) {
-                const float v = acc[bx][by][r];
-                if (v < best[by]) { best[by] = v; bidx[by] = x; }
-              }
-            }
-        } else {
-#pragma unroll
-          for (int bx = 0; bx < 2; ++bx)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int x = xb + bx * 32 + acc_row(r, half);
-#pragma unroll
-              for (int by = 0; by < 2; ++by) {
-                const float v = acc[bx][by][r];
-                if (x < X.rows && v < best[by]) { best[by] = v; bidx[by] = x; }
-              }
-            }
+          for (int by = 0; by < 2; ++by) {
+            const float v = acc[bx][by][r];
+            if (v < best[by]) { best[by] = v; bidx[by] = x; }
+          }
         }
-      }
-      if (more) core.store(lds + ((it + 1) & 1) * C::bufFloats);
-      __syncthreads();
+    } else {
+#pragma unroll
+      for (int bx = 0; bx < 2; ++bx)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int x = xb + bx * 32 + acc_row(r, half);
+#pragma unroll
+          for (int by = 0; by < 2; ++by) {
+            const float v = acc[bx][by][r];
+            if (x < X.rows && v < best[by]) { best[by] = v; bidx[by] = x; }
+          }
+        }
     }
   }
+  __syncthreads();  // the operand buffers are reused below
 
   // the two half-waves hold different x for the same y
 #pragma unroll

@@ -76,34 +76,19 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
   __syncthreads();
 
   C core;
-  const int S = max(1, (a.K + C::KS - 1) / C::KS);
 
   for (int xt0 = xt_begin; xt0 < xt_end; xt0 += kChunkTiles) {
     const int nt = min(kChunkTiles, xt_end - xt0);
-    const int iters = nt * S;
     __syncthreads();  // previous chunk's staging reads are finished
-    core.load(X, Y, xt0 * C::TX, y0, 0, a.K);
-    core.store(lds);
-    __syncthreads();
+    core.begin(X, Y, xt0 * C::TX, y0, a.K, nt, lds);
     f32x16 acc[kChunkTiles][1][1];
-    int it = 0;
 #pragma unroll
     for (int i = 0; i < kChunkTiles; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][0][0][r] = 0.f;
-      if (i < nt) {
-        for (int s = 0; s < S; ++s, ++it) {
-          const bool more = it + 1 < iters;
-          if (more) {
-            const bool wrap = (s + 1 == S);
-            core.load(X, Y, (xt0 + (wrap ? i + 1 : i)) * C::TX, y0, wrap ? 0 : (s + 1) * C::KS, a.K);
-          }
-          core.mma(lds + (it & 1) * C::bufFloats, acc[i]);
-          if (more) core.store(lds + ((it + 1) & 1) * C::bufFloats);
-          __syncthreads();
-        }
-      }
+      if (i < nt) core.tile(X, Y, lds, acc[i]);
     }
+    __syncthreads();  // all fragment reads are done; the buffers become the staging area
 
     // selection, eight rows of the strip per pass
     const int xc0 = xt0 * C::TX;
