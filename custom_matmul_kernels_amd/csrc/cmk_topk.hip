@@ -30,8 +30,7 @@ struct TopkArgs {
   long long strideX, strideY;
   float* values;        // [L][Yext][k]
   long long* indices;   // [L][Yext][k]
-  uint32_t* part_key;   // [splits][L*Yext][128]  (splits > 1)
-  int* part_idx;
+  entry_t* part;        // [splits][L*Yext][128] unordered lists (splits > 1)
   int L, K, k;
   int ystrips, xtiles, splits, tiles_per_split;
 };
@@ -41,10 +40,10 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
   using C = Core<XK, YK, 4, 1, 1, 1>;
   static_assert(C::TX == 128 && C::TY == 32, "tile shape");
   constexpr int opFloats = C::ldsFloats;
-  static_assert(opFloats >= 8 * kStagePitch, "staging area aliases the operand buffers");
+  static_assert(opFloats >= 8 * kStagePitch + 4 * 2 * kTop,
+                "staging area and band lists alias the operand buffers");
   __shared__ __attribute__((aligned(16))) float lds[opFloats];
-  __shared__ uint32_t list_key[32][kTop];
-  __shared__ int list_idx[32][kTop];
+  __shared__ entry_t list[32][kTop];   // running top-128 of every row of the strip
 
   const int total = a.L * a.ystrips * a.splits;
   const int logical = xcd_logical_id(blockIdx.x, total);
@@ -69,11 +68,10 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
   const int half = lane >> 5;
 
   // running lists start empty
-  for (int e = threadIdx.x; e < 32 * kTop; e += kThreads) {
-    (&list_key[0][0])[e] = 0u;
-    (&list_idx[0][0])[e] = -1;
-  }
+  for (int e = threadIdx.x; e < 32 * kTop; e += kThreads) (&list[0][0])[e] = 0ull;
   __syncthreads();
+  entry_t* band = reinterpret_cast<entry_t*>(lds + 8 * kStagePitch) + wave * kTop;
+  uint32_t seed = 0;
 
   C core;
 
@@ -119,13 +117,23 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
           const int x = xc0 + lane + 64 * j;
           const bool ok = x < x_limit;
           key[j] = ok ? f2key(src[lane + 64 * j]) : 0u;
-          idx[j] = ok ? x : -1;
+          idx[j] = x;
         }
-        key[16] = list_key[r][lane];
-        idx[16] = list_idx[r][lane];
-        key[17] = list_key[r][lane + 64];
-        idx[17] = list_idx[r][lane + 64];
-        select128<18>(key, idx, list_key[r], list_idx[r]);
+        if (xt0 == xt_begin) {
+          // first chunk: the running list is empty
+          uint32_t k16[16];
+          int i16[16];
+#pragma unroll
+          for (int j = 0; j < 16; ++j) { k16[j] = key[j]; i16[j] = idx[j]; }
+          select128<16>(k16, i16, seed, band, list[r]);
+        } else {
+          const entry_t r0 = list[r][lane], r1 = list[r][lane + 64];
+          key[16] = entry_key(r0);
+          idx[16] = entry_idx(r0);
+          key[17] = entry_key(r1);
+          idx[17] = entry_idx(r1);
+          select128<18>(key, idx, seed, band, list[r]);
+        }
       }
     }
   }
@@ -140,13 +148,11 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
       if (y >= Yext) continue;
       const long long orow = (long long)b * Yext + y;
       if (a.splits == 1) {
-        sort_and_store(list_key[r], list_idx[r], a.values + orow * a.k, a.indices + orow * a.k, a.k);
+        sort_and_store(list[r], a.values + orow * a.k, a.indices + orow * a.k, a.k);
       } else {
         const long long o = ((long long)split * a.L * Yext + orow) * kTop;
-        a.part_key[o + lane] = list_key[r][lane];
-        a.part_idx[o + lane] = list_idx[r][lane];
-        a.part_key[o + lane + 64] = list_key[r][lane + 64];
-        a.part_idx[o + lane + 64] = list_idx[r][lane + 64];
+        a.part[o + lane] = list[r][lane];
+        a.part[o + lane + 64] = list[r][lane + 64];
       }
     }
   }
@@ -154,56 +160,52 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
 
 // One wave per output row: folds `parts` unordered 128-entry lists into one,
 // orders it and stores the first k entries.
-__global__ __launch_bounds__(kThreads) void topk_merge_kernel(const uint32_t* part_key,
-                                                              const int* part_idx, float* values,
+__global__ __launch_bounds__(kThreads) void topk_merge_kernel(const entry_t* part, float* values,
                                                               long long* indices, long long rows,
                                                               int parts, int k) {
-  __shared__ uint32_t list_key[4][kTop];
-  __shared__ int list_idx[4][kTop];
+  __shared__ entry_t list[4][kTop];
+  __shared__ entry_t bands[4][kTop];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const long long row = (long long)blockIdx.x * 4 + wave;
   if (row >= rows) return;
-  list_key[wave][lane] = 0u;
-  list_key[wave][lane + 64] = 0u;
-  list_idx[wave][lane] = -1;
-  list_idx[wave][lane + 64] = -1;
+  list[wave][lane] = 0ull;
+  list[wave][lane + 64] = 0ull;
+  uint32_t seed = 0;
   for (int p0 = 0; p0 < parts; p0 += 8) {
     uint32_t key[18];
     int idx[18];
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       const int p = p0 + (j >> 1);
-      const bool ok = p < parts;
-      const long long o = ((long long)p * rows + row) * kTop + lane + 64 * (j & 1);
-      key[j] = ok ? part_key[o] : 0u;
-      idx[j] = ok ? part_idx[o] : -1;
+      const entry_t e = p < parts ? part[((long long)p * rows + row) * kTop + lane + 64 * (j & 1)] : 0ull;
+      key[j] = entry_key(e);
+      idx[j] = entry_idx(e);
     }
-    key[16] = list_key[wave][lane];
-    idx[16] = list_idx[wave][lane];
-    key[17] = list_key[wave][lane + 64];
-    idx[17] = list_idx[wave][lane + 64];
-    select128<18>(key, idx, list_key[wave], list_idx[wave]);
+    const entry_t r0 = list[wave][lane], r1 = list[wave][lane + 64];
+    key[16] = entry_key(r0);
+    idx[16] = entry_idx(r0);
+    key[17] = entry_key(r1);
+    idx[17] = entry_idx(r1);
+    select128<18>(key, idx, seed, bands[wave], list[wave]);
   }
-  sort_and_store(list_key[wave], list_idx[wave], values + row * k, indices + row * k, k);
+  sort_and_store(list[wave], values + row * k, indices + row * k, k);
 }
 
 // One wave per part of a 1-D array: keeps the best 128 of its range.
 __global__ __launch_bounds__(kThreads) void topk1d_partial_kernel(const float* arr, long long n,
                                                                   long long span, int parts,
-                                                                  uint32_t* part_key,
-                                                                  int* part_idx) {
-  __shared__ uint32_t list_key[4][kTop];
-  __shared__ int list_idx[4][kTop];
+                                                                  entry_t* part) {
+  __shared__ entry_t list[4][kTop];
+  __shared__ entry_t bands[4][kTop];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int part = blockIdx.x * 4 + wave;
-  if (part >= parts) return;
-  list_key[wave][lane] = 0u;
-  list_key[wave][lane + 64] = 0u;
-  list_idx[wave][lane] = -1;
-  list_idx[wave][lane + 64] = -1;
-  const long long begin = (long long)part * span;
+  const int p = blockIdx.x * 4 + wave;
+  if (p >= parts) return;
+  list[wave][lane] = 0ull;
+  list[wave][lane + 64] = 0ull;
+  uint32_t seed = 0;
+  const long long begin = (long long)p * span;
   const long long end = begin + span < n ? begin + span : n;
   for (long long c0 = begin; c0 < end; c0 += 1024) {
     uint32_t key[18];
@@ -213,19 +215,18 @@ __global__ __launch_bounds__(kThreads) void topk1d_partial_kernel(const float* a
       const long long x = c0 + lane + 64 * j;
       const bool ok = x < end;
       key[j] = ok ? f2key(arr[x]) : 0u;
-      idx[j] = ok ? (int)x : -1;
+      idx[j] = (int)x;
     }
-    key[16] = list_key[wave][lane];
-    idx[16] = list_idx[wave][lane];
-    key[17] = list_key[wave][lane + 64];
-    idx[17] = list_idx[wave][lane + 64];
-    select128<18>(key, idx, list_key[wave], list_idx[wave]);
+    const entry_t r0 = list[wave][lane], r1 = list[wave][lane + 64];
+    key[16] = entry_key(r0);
+    idx[16] = entry_idx(r0);
+    key[17] = entry_key(r1);
+    idx[17] = entry_idx(r1);
+    select128<18>(key, idx, seed, bands[wave], list[wave]);
   }
-  const long long o = (long long)part * kTop;
-  part_key[o + lane] = list_key[wave][lane];
-  part_idx[o + lane] = list_idx[wave][lane];
-  part_key[o + lane + 64] = list_key[wave][lane + 64];
-  part_idx[o + lane + 64] = list_idx[wave][lane + 64];
+  const long long o = (long long)p * kTop;
+  part[o + lane] = list[wave][lane];
+  part[o + lane + 64] = list[wave][lane + 64];
 }
 
 static void plan_topk(int L, int Xext, int Yext, int* ystrips, int* xtiles, int* splits,
@@ -306,8 +307,7 @@ extern "C" int cmk_topk_bmm_f32(const float* A, const float* B, float* values, l
     if (!workspace || workspace_bytes < need)
       return fail(CMK_ERR_WORKSPACE, "cmk_topk_bmm_f32: workspace of %zu bytes required, %zu given",
                   need, workspace_bytes);
-    a.part_key = static_cast<uint32_t*>(workspace);
-    a.part_idx = reinterpret_cast<int*>(a.part_key + (size_t)a.splits * d->L * Yext * kTop);
+    a.part = static_cast<entry_t*>(workspace);
   }
   const long long total = (long long)d->L * a.ystrips * a.splits;
   if (int e = check_grid(total)) return e;
@@ -322,7 +322,7 @@ extern "C" int cmk_topk_bmm_f32(const float* A, const float* B, float* values, l
     const long long rows = (long long)d->L * Yext;
     if (int e = check_grid((rows + 3) / 4)) return e;
     hipLaunchKernelGGL(topk_merge_kernel, dim3((unsigned)((rows + 3) / 4)), block, 0, st,
-                       a.part_key, a.part_idx, values, indices, rows, a.splits, k);
+                       a.part, values, indices, rows, a.splits, k);
     if (int e = hip_status(hipGetLastError(), "cmk_topk_bmm_f32 merge launch")) return e;
   }
   return CMK_OK;
@@ -341,13 +341,12 @@ extern "C" int cmk_topk_1d_f32(const float* arr, long long n, float* values, lon
   if (!workspace || workspace_bytes < need)
     return fail(CMK_ERR_WORKSPACE, "cmk_topk_1d_f32: workspace of %zu bytes required, %zu given",
                 need, workspace_bytes);
-  uint32_t* pk = static_cast<uint32_t*>(workspace);
-  int* pi = reinterpret_cast<int*>(pk + (size_t)parts * kTop);
+  entry_t* part = static_cast<entry_t*>(workspace);
   hipStream_t st = (hipStream_t)stream;
   hipLaunchKernelGGL(topk1d_partial_kernel, dim3((unsigned)((parts + 3) / 4)), dim3(kThreads), 0, st,
-                     arr, n, span, parts, pk, pi);
+                     arr, n, span, parts, part);
   if (int e = hip_status(hipGetLastError(), "cmk_topk_1d_f32 launch")) return e;
-  hipLaunchKernelGGL(topk_merge_kernel, dim3(1), dim3(kThreads), 0, st, pk, pi, values, indices,
+  hipLaunchKernelGGL(topk_merge_kernel, dim3(1), dim3(kThreads), 0, st, part, values, indices,
                      (long long)1, parts, k);
   return hip_status(hipGetLastError(), "cmk_topk_1d_f32 merge launch");
 }
