@@ -74,8 +74,8 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
     }
   }
 
-  Operand X{a.A + (long long)b * a.strideA, a.lda, a.M, a.vecA};
-  Operand Y{a.B + (long long)b * a.strideB, a.ldb, a.N, a.vecB};
+  Operand X{uniform_ptr(a.A + (long long)b * a.strideA), a.lda, a.M, a.vecA};
+  Operand Y{uniform_ptr(a.B + (long long)b * a.strideB), a.ldb, a.N, a.vecB};
 
   C core;
   f32x16 acc[2][2];

@@ -34,6 +34,12 @@ namespace cmk {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+// Operands live in global memory; loading through pointers that say so gives
+// global_load instructions (a generic pointer would give flat loads, which
+// also count against the LDS wait counter).
+typedef const f32x4 __attribute__((address_space(1))) * global_f32x4_ptr;
+typedef const float __attribute__((address_space(1))) * global_f32_ptr;
+
 constexpr int kThreads = 256;
 constexpr int KC = 0;   // k-contiguous operand
 constexpr int RC = 1;   // row-contiguous operand
@@ -44,6 +50,16 @@ struct Operand {
   int rows;        // extent of the non-contracted axis
   int vec;         // non-zero when 16-byte loads are legal (base and ld aligned)
 };
+
+// Marks a pointer that is the same for every lane of the wave as such, so that
+// address arithmetic on it stays on the scalar unit.
+template <class P>
+__device__ __forceinline__ P* uniform_ptr(P* p) {
+  const unsigned long long v = reinterpret_cast<unsigned long long>(p);
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
+  return reinterpret_cast<P*>((static_cast<unsigned long long>(hi) << 32) | lo);
+}
 
 // LDS footprint of one slab (KS deep) of a T-row operand tile.
 template <int KIND, int T, int KS>
@@ -60,33 +76,55 @@ struct TileLayout<RC, T, KS> {
 };
 
 // ---- global -> registers ---------------------------------------------------
-// Each thread fetches NV = T*KS/1024 groups of four consecutive floats.  A tile
-// that lies completely inside the matrix takes the branch-free path.
+// Each thread fetches NV = T*KS/1024 groups of four consecutive floats.  For
+// both kinds the element a thread fetches in pass p sits at
+//     tile + (t / TPR + p * RPP) * ld + (t % TPR) * 4
+// (KC: row-major rows x k, RC: k-major k x rows), so the per-lane part
+// `lane_off` is fixed for a whole kernel and everything else is scalar.
 template <int KIND, int T, int KS>
-__device__ __forceinline__ void gload(const Operand& o, int r0, int k0, int K,
-                                      f32x4 (&v)[T * KS / 1024]) {
-  constexpr int NV = T * KS / 1024;
+struct LoadMap {
+  static constexpr int NV = T * KS / 1024;
+  static constexpr int TPR = KIND == KC ? KS / 4 : T / 4;  // threads per contiguous run
+  static constexpr int RPP = kThreads / TPR;               // runs per pass
+};
+
+template <int KIND, int T, int KS>
+__device__ __forceinline__ void lane_offsets_bytes(const Operand& o,
+                                                   unsigned (&off)[T * KS / 1024]) {
+  using M = LoadMap<KIND, T, KS>;
   const int t = threadIdx.x;
-  const bool interior = o.vec && (k0 + KS <= K) && (r0 + T <= o.rows);  // uniform
-  if constexpr (KIND == KC) {
-    constexpr int TPR = KS / 4;          // threads per row
-    constexpr int RPP = kThreads / TPR;  // rows per pass
-    const int kk = k0 + (t % TPR) * 4;
-    const int rr = r0 + t / TPR;
-    if (interior) {
-      const float* src = o.p + (long long)rr * o.ld + kk;
 #pragma unroll
-      for (int p = 0; p < NV; ++p)
-        v[p] = *reinterpret_cast<const f32x4*>(src + (long long)p * RPP * o.ld);
-    } else if (K > 0 && o.rows > 0) {
-      // edge tile: every element is fetched from a clamped (always valid)
-      // address and zeroed when it lies outside the matrix; no divergent branches
+  for (int p = 0; p < M::NV; ++p)
+    off[p] = static_cast<unsigned>(((long long)(t / M::TPR + p * M::RPP) * o.ld + (t % M::TPR) * 4) * 4);
+}
+
+// r0, k0, K are wave-uniform.  A tile that lies completely inside the matrix
+// takes the branch-free path.
+template <int KIND, int T, int KS>
+__device__ __forceinline__ void gload(const Operand& o, const unsigned (&lane_off)[T * KS / 1024],
+                                      int r0, int k0, int K, f32x4 (&v)[T * KS / 1024]) {
+  using M = LoadMap<KIND, T, KS>;
+  constexpr int NV = M::NV, TPR = M::TPR, RPP = M::RPP;
+  const int t = threadIdx.x;
+  const bool interior = o.vec && (k0 + KS <= K) && (r0 + T <= o.rows) &&
+                        ((long long)(T + KS) * o.ld < (1ll << 29));
+  if (interior) {
+    const long long first = KIND == KC ? (long long)r0 * o.ld + k0 : (long long)k0 * o.ld + r0;
+    const char* tile = reinterpret_cast<const char*>(o.p + first);
+#pragma unroll
+    for (int p = 0; p < NV; ++p) v[p] = *(global_f32x4_ptr)(tile + lane_off[p]);
+  } else if (K > 0 && o.rows > 0) {
+    // edge tile: every element is fetched from a clamped (always valid)
+    // address and zeroed when it lies outside the matrix; no divergent branches
+    if constexpr (KIND == KC) {
+      const int kk = k0 + (t % TPR) * 4;
+      const int rr = r0 + t / TPR;
 #pragma unroll
       for (int p = 0; p < NV; ++p) {
         const int row = rr + RPP * p;
         const float* src = o.p + (long long)row * o.ld + kk;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) v[p][j] = *((row < o.rows && kk + j < K) ? src + j : o.p);
+        for (int j = 0; j < 4; ++j) v[p][j] = *(global_f32_ptr)((row < o.rows && kk + j < K) ? src + j : o.p);
       }
 #pragma unroll
       for (int p = 0; p < NV; ++p) {
@@ -95,26 +133,14 @@ __device__ __forceinline__ void gload(const Operand& o, int r0, int k0, int K,
         for (int j = 0; j < 4; ++j) v[p][j] = (row < o.rows && kk + j < K) ? v[p][j] : 0.f;
       }
     } else {
-#pragma unroll
-      for (int p = 0; p < NV; ++p) v[p] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-  } else {
-    constexpr int TPR = T / 4;           // threads per k-row
-    constexpr int RPP = kThreads / TPR;  // k-rows per pass
-    const int rr = r0 + (t % TPR) * 4;
-    const int kb = k0 + t / TPR;
-    if (interior) {
-      const float* src = o.p + (long long)kb * o.ld + rr;
-#pragma unroll
-      for (int p = 0; p < NV; ++p)
-        v[p] = *reinterpret_cast<const f32x4*>(src + (long long)p * RPP * o.ld);
-    } else if (K > 0 && o.rows > 0) {
+      const int rr = r0 + (t % TPR) * 4;
+      const int kb = k0 + t / TPR;
 #pragma unroll
       for (int p = 0; p < NV; ++p) {
         const int kk = kb + p * RPP;
         const float* src = o.p + (long long)kk * o.ld + rr;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) v[p][j] = *((kk < K && rr + j < o.rows) ? src + j : o.p);
+        for (int j = 0; j < 4; ++j) v[p][j] = *(global_f32_ptr)((kk < K && rr + j < o.rows) ? src + j : o.p);
       }
 #pragma unroll
       for (int p = 0; p < NV; ++p) {
@@ -122,24 +148,22 @@ __device__ __forceinline__ void gload(const Operand& o, int r0, int k0, int K,
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[p][j] = (kk < K && rr + j < o.rows) ? v[p][j] : 0.f;
       }
-    } else {
-#pragma unroll
-      for (int p = 0; p < NV; ++p) v[p] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+  } else {
+#pragma unroll
+    for (int p = 0; p < NV; ++p) v[p] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 }
 
 // ---- registers -> LDS --------------------------------------------------------
 template <int KIND, int T, int KS>
 __device__ __forceinline__ void lstore(float* lds, const f32x4 (&v)[T * KS / 1024]) {
-  constexpr int NV = T * KS / 1024;
+  using M = LoadMap<KIND, T, KS>;
   const int t = threadIdx.x;
   constexpr int pitch = TileLayout<KIND, T, KS>::pitch;
-  constexpr int TPR = KIND == KC ? KS / 4 : T / 4;
-  constexpr int RPP = kThreads / TPR;
 #pragma unroll
-  for (int p = 0; p < NV; ++p)
-    *reinterpret_cast<f32x4*>(&lds[(t / TPR + p * RPP) * pitch + (t % TPR) * 4]) = v[p];
+  for (int p = 0; p < M::NV; ++p)
+    *reinterpret_cast<f32x4*>(&lds[(t / M::TPR + p * M::RPP) * pitch + (t % M::TPR) * 4]) = v[p];
 }
 
 // ---- LDS -> MFMA fragment ----------------------------------------------------
@@ -189,14 +213,20 @@ struct Core {
   f32x4 yv[TY * KS / 1024];
   f32x4 xf[2][BX];           // fragments; [0] holds k-group 0 of the current slab at slab entry
   f32x4 yf[2][BY];
-  int it, iters, S;          // flat slab counter
-  int lt, ls;                // (tile, slab) of the next slab to fetch
+  int it, iters, S;          // flat slab counter (wave-uniform)
+  int lt, ls;                // (tile, slab) of the next slab to fetch (wave-uniform)
   int xbase, y0, K;
   int xr, yr, half;
+  unsigned xoff[TX * KS / 1024];  // this lane's byte offsets inside an operand tile
+  unsigned yoff[TY * KS / 1024];
 
   __device__ __forceinline__ void load(const Operand& X, const Operand& Y) {
-    gload<XK, TX, KS>(X, xbase + lt * TX, ls * KS, K, xv);
-    gload<YK, TY, KS>(Y, y0, ls * KS, K, yv);
+    // the slab coordinates are the same for every lane; saying so keeps the
+    // address arithmetic on the scalar unit
+    const int x0 = __builtin_amdgcn_readfirstlane(xbase + lt * TX);
+    const int k0 = __builtin_amdgcn_readfirstlane(ls * KS);
+    gload<XK, TX, KS>(X, xoff, x0, k0, K, xv);
+    gload<YK, TY, KS>(Y, yoff, y0, k0, K, yv);
     if (++ls == S) { ls = 0; ++lt; }
   }
   __device__ __forceinline__ void store(float* buf) {
@@ -220,11 +250,13 @@ struct Core {
     half = lane >> 5;
     xr = (wave % WX) * BX * 32 + (lane & 31);
     yr = (wave / WX) * BY * 32 + (lane & 31);
-    xbase = xbase_;
-    y0 = y0_;
-    K = K_;
+    xbase = __builtin_amdgcn_readfirstlane(xbase_);
+    y0 = __builtin_amdgcn_readfirstlane(y0_);
+    K = __builtin_amdgcn_readfirstlane(K_);
     S = max(1, (K + KS - 1) / KS);
-    iters = ntiles * S;
+    iters = __builtin_amdgcn_readfirstlane(ntiles) * S;
+    lane_offsets_bytes<XK, TX, KS>(X, xoff);
+    lane_offsets_bytes<YK, TY, KS>(Y, yoff);
     it = 0;
     lt = 0;
     ls = 0;

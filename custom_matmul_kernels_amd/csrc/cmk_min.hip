@@ -56,8 +56,8 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
   const int xt_end = min(a.xtiles, xt_begin + a.tiles_per_split);
 
   Operand X = a.X, Y = a.Y;
-  X.p += (long long)b * a.strideX;
-  Y.p += (long long)b * a.strideY;
+  X.p = uniform_ptr(X.p + (long long)b * a.strideX);
+  Y.p = uniform_ptr(Y.p + (long long)b * a.strideY);
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;

@@ -57,8 +57,8 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
   const int xt_end = min(a.xtiles, xt_begin + a.tiles_per_split);
 
   Operand X = a.X, Y = a.Y;
-  X.p += (long long)b * a.strideX;
-  Y.p += (long long)b * a.strideY;
+  X.p = uniform_ptr(X.p + (long long)b * a.strideX);
+  Y.p = uniform_ptr(Y.p + (long long)b * a.strideY);
   const int x_limit = min(X.rows, xt_end * C::TX);
   const int Yext = Y.rows;
 
@@ -71,7 +71,7 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
   for (int e = threadIdx.x; e < 32 * kTop; e += kThreads) (&list[0][0])[e] = 0ull;
   __syncthreads();
   entry_t* band = reinterpret_cast<entry_t*>(lds + 8 * kStagePitch) + wave * kTop;
-  uint32_t seed = 0;
+  uint32_t seed[1] = {0u};
 
   C core;
 
@@ -109,50 +109,58 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
       for (int rr = 0; rr < 2; ++rr) {
         const int r = 8 * g + 2 * wave + rr;  // row of the strip, owned by this wave
         if (y0 + r >= Yext) continue;
+        entry_t* const outs[1] = {list[r]};
+        entry_t* const bands[1] = {band};
         const float* src = lds + (r & 7) * kStagePitch;
-        uint32_t key[18];
-        int idx[18];
+        const int xl = xc0 + lane;
+        uint32_t key[1][18];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const int x = xc0 + lane + 64 * j;
-          const bool ok = x < x_limit;
-          key[j] = ok ? f2key(src[lane + 64 * j]) : 0u;
-          idx[j] = x;
-        }
+        for (int j = 0; j < 16; ++j)
+          key[0][j] = xl + 64 * j < x_limit ? f2key(src[lane + 64 * j]) : 0u;
         if (xt0 == xt_begin) {
           // first chunk: the running list is empty
-          uint32_t k16[16];
-          int i16[16];
+          uint32_t k16[1][16];
 #pragma unroll
-          for (int j = 0; j < 16; ++j) { k16[j] = key[j]; i16[j] = idx[j]; }
-          select128<16>(k16, i16, seed, band, list[r]);
+          for (int j = 0; j < 16; ++j) k16[0][j] = key[0][j];
+          select128<16, 1>(k16, [&](int, int j) { return xl + 64 * j; }, seed, bands, outs);
         } else {
-          const entry_t r0 = list[r][lane], r1 = list[r][lane + 64];
-          key[16] = entry_key(r0);
-          idx[16] = entry_idx(r0);
-          key[17] = entry_key(r1);
-          idx[17] = entry_idx(r1);
-          select128<18>(key, idx, seed, band, list[r]);
+          const entry_t e0 = list[r][lane], e1 = list[r][lane + 64];
+          key[0][16] = entry_key(e0);
+          key[0][17] = entry_key(e1);
+          const int ri0 = entry_idx(e0), ri1 = entry_idx(e1);
+          select128<18, 1>(key, [&](int, int j) { return j < 16 ? xl + 64 * j : (j == 16 ? ri0 : ri1); },
+                           seed, bands, outs);
         }
       }
     }
   }
 
-  // each wave finishes the rows it owns
+  // each wave finishes the rows it owns, two at a time
 #pragma unroll 1
   for (int g = 0; g < 4; ++g) {
-#pragma unroll 1
-    for (int rr = 0; rr < 2; ++rr) {
-      const int r = 8 * g + 2 * wave + rr;
-      const int y = y0 + r;
-      if (y >= Yext) continue;
-      const long long orow = (long long)b * Yext + y;
-      if (a.splits == 1) {
-        sort_and_store(list[r], a.values + orow * a.k, a.indices + orow * a.k, a.k);
-      } else {
-        const long long o = ((long long)split * a.L * Yext + orow) * kTop;
-        a.part[o + lane] = list[r][lane];
-        a.part[o + lane + 64] = list[r][lane + 64];
+    const int r0 = 8 * g + 2 * wave;
+    if (a.splits == 1) {
+      const entry_t* const lists[2] = {list[r0], list[r0 + 1]};
+      float* vals[2];
+      long long* inds[2];
+#pragma unroll
+      for (int rr = 0; rr < 2; ++rr) {
+        const int y = y0 + r0 + rr;
+        const long long orow = (long long)b * Yext + y;
+        vals[rr] = y < Yext ? a.values + orow * a.k : nullptr;
+        inds[rr] = y < Yext ? a.indices + orow * a.k : nullptr;
+      }
+      float* const cv[2] = {vals[0], vals[1]};
+      long long* const ci[2] = {inds[0], inds[1]};
+      sort_and_store<2>(lists, cv, ci, a.k);
+    } else {
+#pragma unroll
+      for (int rr = 0; rr < 2; ++rr) {
+        const int y = y0 + r0 + rr;
+        if (y >= Yext) continue;
+        const long long o = ((long long)split * a.L * Yext + (long long)b * Yext + y) * kTop;
+        a.part[o + lane] = list[r0 + rr][lane];
+        a.part[o + lane + 64] = list[r0 + rr][lane + 64];
       }
     }
   }
@@ -171,25 +179,30 @@ __global__ __launch_bounds__(kThreads) void topk_merge_kernel(const entry_t* par
   if (row >= rows) return;
   list[wave][lane] = 0ull;
   list[wave][lane + 64] = 0ull;
-  uint32_t seed = 0;
+  uint32_t seed[1] = {0u};
+  entry_t* const outs[1] = {list[wave]};
+  entry_t* const bnds[1] = {bands[wave]};
   for (int p0 = 0; p0 < parts; p0 += 8) {
-    uint32_t key[18];
-    int idx[18];
+    uint32_t key[1][18];
+    int idx[1][18];
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       const int p = p0 + (j >> 1);
       const entry_t e = p < parts ? part[((long long)p * rows + row) * kTop + lane + 64 * (j & 1)] : 0ull;
-      key[j] = entry_key(e);
-      idx[j] = entry_idx(e);
+      key[0][j] = entry_key(e);
+      idx[0][j] = entry_idx(e);
     }
     const entry_t r0 = list[wave][lane], r1 = list[wave][lane + 64];
-    key[16] = entry_key(r0);
-    idx[16] = entry_idx(r0);
-    key[17] = entry_key(r1);
-    idx[17] = entry_idx(r1);
-    select128<18>(key, idx, seed, bands[wave], list[wave]);
+    key[0][16] = entry_key(r0);
+    idx[0][16] = entry_idx(r0);
+    key[0][17] = entry_key(r1);
+    idx[0][17] = entry_idx(r1);
+    select128<18, 1>(key, [&](int, int j) { return idx[0][j]; }, seed, bnds, outs);
   }
-  sort_and_store(list[wave], values + row * k, indices + row * k, k);
+  const entry_t* const lists[1] = {list[wave]};
+  float* const cv[1] = {values + row * k};
+  long long* const ci[1] = {indices + row * k};
+  sort_and_store<1>(lists, cv, ci, k);
 }
 
 // One wave per part of a 1-D array: keeps the best 128 of its range.
@@ -204,25 +217,27 @@ __global__ __launch_bounds__(kThreads) void topk1d_partial_kernel(const float* a
   if (p >= parts) return;
   list[wave][lane] = 0ull;
   list[wave][lane + 64] = 0ull;
-  uint32_t seed = 0;
+  uint32_t seed[1] = {0u};
+  entry_t* const outs[1] = {list[wave]};
+  entry_t* const bnds[1] = {bands[wave]};
   const long long begin = (long long)p * span;
   const long long end = begin + span < n ? begin + span : n;
   for (long long c0 = begin; c0 < end; c0 += 1024) {
-    uint32_t key[18];
-    int idx[18];
+    uint32_t key[1][18];
+    int idx[1][18];
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       const long long x = c0 + lane + 64 * j;
       const bool ok = x < end;
-      key[j] = ok ? f2key(arr[x]) : 0u;
-      idx[j] = (int)x;
+      key[0][j] = ok ? f2key(arr[x]) : 0u;
+      idx[0][j] = (int)x;
     }
     const entry_t r0 = list[wave][lane], r1 = list[wave][lane + 64];
-    key[16] = entry_key(r0);
-    idx[16] = entry_idx(r0);
-    key[17] = entry_key(r1);
-    idx[17] = entry_idx(r1);
-    select128<18>(key, idx, seed, bands[wave], list[wave]);
+    key[0][16] = entry_key(r0);
+    idx[0][16] = entry_idx(r0);
+    key[0][17] = entry_key(r1);
+    idx[0][17] = entry_idx(r1);
+    select128<18, 1>(key, [&](int, int j) { return idx[0][j]; }, seed, bnds, outs);
   }
   const long long o = (long long)p * kTop;
   part[o + lane] = list[wave][lane];
