@@ -18,7 +18,8 @@ struct BmmArgs {
   const uint8_t* element_mask;
   long long lda, ldb, strideA, strideB;
   int L, M, N, K;
-  int tiles_m, tiles_n, group_m;
+  int tiles_m, tiles_n;
+  int run;           // consecutive tiles along m per work-group
   int mask_batched;  // 1: masks have a leading batch axis, 0: shared by all batches
   int vecA, vecB;
 };
@@ -28,21 +29,22 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
   using C = Core<XK, YK, 2, 2, 2, 2>;
   __shared__ __attribute__((aligned(16))) float lds[C::ldsFloats];
 
-  const int tiles = a.tiles_m * a.tiles_n;
-  const int logical = xcd_logical_id(blockIdx.x, a.L * tiles);
+  // A work-group owns `run` consecutive tiles along m of one 128-wide column
+  // strip; the slab pipeline runs across them, so the stores of one tile
+  // overlap the loads of the next.  Masked products use run == 1 because
+  // skipped tiles break the sequence.
+  const int mgroups = (a.tiles_m + a.run - 1) / a.run;
+  const int per_batch = mgroups * a.tiles_n;
+  const int logical = xcd_logical_id(blockIdx.x, a.L * per_batch);
   if (logical < 0) return;
-  const int b = logical / tiles;
-  const int t = logical - b * tiles;
-  // grouped rasterisation: walk group_m tile-rows together so that concurrently
-  // running work-groups share panels of A and B in L2
-  const int per_group = a.group_m * a.tiles_n;
-  const int g = t / per_group;
-  const int first_m = g * a.group_m;
-  const int gsz = min(a.tiles_m - first_m, a.group_m);
-  const int in_g = t - g * per_group;
-  const int tile_m = first_m + in_g % gsz;
-  const int tile_n = in_g / gsz;
-  const int m0 = tile_m * C::TX;
+  const int b = logical / per_batch;
+  const int t = logical - b * per_batch;
+  // column strips of one row group are neighbours, so that concurrently
+  // running work-groups share their panels of A in L2
+  const int mg = t / a.tiles_n;
+  const int tile_n = t - mg * a.tiles_n;
+  const int tile_m0 = mg * a.run;
+  const int ntiles = min(a.run, a.tiles_m - tile_m0);
   const int n0 = tile_n * C::TY;
 
   const int lane = threadIdx.x & 63;
@@ -54,9 +56,10 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
   long long mb = 0;  // batch index into the masks
   if constexpr (MASKED) {
     mb = a.mask_batched ? b : 0;
-    const uint8_t bm = a.block_mask[(mb * a.tiles_m + tile_m) * a.tiles_n + tile_n];
+    const uint8_t bm = a.block_mask[(mb * a.tiles_m + tile_m0) * a.tiles_n + tile_n];
     if (bm == 0) {
       // skipped tile: nothing is loaded or multiplied, zeros are written
+      const int m0 = tile_m0 * C::TX;
       for (int e = threadIdx.x; e < 128 * 32; e += kThreads) {
         const int r = m0 + (e >> 5);
         const int c = n0 + (e & 31) * 4;
@@ -78,38 +81,86 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
   Operand Y{uniform_ptr(a.B + (long long)b * a.strideB), a.ldb, a.N, a.vecB};
 
   C core;
-  f32x16 acc[2][2];
+  core.begin(X, Y, tile_m0 * C::TX, n0, a.K, ntiles, lds);
+  for (int ti = 0; ti < ntiles; ++ti) {
+    f32x16 acc[2][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    core.tile(X, Y, lds, acc);
 
-  core.begin(X, Y, m0, n0, a.K, 1, lds);
-  core.tile(X, Y, lds, acc);
-
-  // epilogue
-  const int mw = m0 + (wave % 2) * 64;
-  const int nw = n0 + (wave / 2) * 64;
+    // store: one accumulator register covers two 128-byte row segments of C
+    const int wv = __builtin_amdgcn_readfirstlane(wave);
+    const int mw = (tile_m0 + ti) * C::TX + (wv % 2) * 64;
+    const int nw = n0 + (wv / 2) * 64;
+    if (mw + 64 <= a.M && nw + 64 <= a.N && (long long)a.N * 68 * 4 < (1ll << 31)) {
+      // interior: row addresses are scalar, the lane part is one 32-bit offset
+      typedef float __attribute__((address_space(1))) * gfp;
+      typedef const uint8_t __attribute__((address_space(1))) * gbp;
+      char* base = reinterpret_cast<char*>(uniform_ptr(Cb + (long long)mw * a.N + nw));
+      const unsigned voff = static_cast<unsigned>((4 * half * a.N + l32) * 4);
+      if constexpr (!MASKED) {
 #pragma unroll
-  for (int bx = 0; bx < 2; ++bx) {
+        for (int bx = 0; bx < 2; ++bx)
 #pragma unroll
-    for (int by = 0; by < 2; ++by) {
-      const int n = nw + by * 32 + l32;
+          for (int r = 0; r < 16; ++r) {
+            char* rp = base + (long long)(bx * 32 + 8 * (r >> 2) + (r & 3)) * a.N * 4;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = mw + bx * 32 + acc_row(r, half);
-        if (m < a.M && n < a.N) {
-          float v = acc[bx][by][r];
-          if constexpr (MASKED) {
-            const int tn8 = (a.N + 7) >> 3;
-            const int tm8 = (a.M + 7) >> 3;
-            const uint8_t tm = a.thread_mask[(mb * tm8 + (m >> 3)) * tn8 + (n >> 3)];
-            const uint8_t em = a.element_mask[(mb * a.M + m) * a.N + n];
-            v = tm ? v * (float)em : 0.f;
+            for (int by = 0; by < 2; ++by) *(gfp)(rp + voff + by * 128) = acc[bx][by][r];
           }
-          Cb[(long long)m * a.N + n] = v;
+      } else {
+        const int tn8 = (a.N + 7) >> 3;
+        const int tm8 = (a.M + 7) >> 3;
+        const uint8_t* eb = uniform_ptr(a.element_mask + (mb * a.M + mw) * a.N + nw);
+        const uint8_t* tb = uniform_ptr(a.thread_mask + (mb * tm8 + (mw >> 3)) * tn8 + (nw >> 3));
+        const unsigned eoff = static_cast<unsigned>(4 * half * a.N + l32);
+        const unsigned toff = static_cast<unsigned>(l32 >> 3);
+#pragma unroll
+        for (int bx = 0; bx < 2; ++bx)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            uint8_t tmk[2];
+#pragma unroll
+            for (int by = 0; by < 2; ++by)
+              tmk[by] = *(gbp)(tb + (long long)(bx * 4 + q) * tn8 + toff + by * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int r = 4 * q + e;
+              const long long rowc = bx * 32 + 8 * q + e;
+              char* rp = base + rowc * a.N * 4;
+              const uint8_t* ep = eb + rowc * a.N;
+#pragma unroll
+              for (int by = 0; by < 2; ++by) {
+                const uint8_t em = *(gbp)(ep + eoff + by * 32);
+                *(gfp)(rp + voff + by * 128) = tmk[by] ? acc[bx][by][r] * (float)em : 0.f;
+              }
+            }
+          }
+      }
+    } else {
+#pragma unroll
+      for (int bx = 0; bx < 2; ++bx) {
+#pragma unroll
+        for (int by = 0; by < 2; ++by) {
+          const int n = nw + by * 32 + l32;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int m = mw + bx * 32 + acc_row(r, half);
+            if (m < a.M && n < a.N) {
+              float v = acc[bx][by][r];
+              if constexpr (MASKED) {
+                const int tn8 = (a.N + 7) >> 3;
+                const int tm8 = (a.M + 7) >> 3;
+                const uint8_t tm = a.thread_mask[(mb * tm8 + (m >> 3)) * tn8 + (n >> 3)];
+                const uint8_t em = a.element_mask[(mb * a.M + m) * a.N + n];
+                v = tm ? v * (float)em : 0.f;
+              }
+              Cb[(long long)m * a.N + n] = v;
+            }
+          }
         }
       }
     }
@@ -118,7 +169,7 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
 
 template <bool MASKED>
 static hipError_t launch_bmm(const BmmArgs& a, int transA, int transB, hipStream_t st) {
-  const int total = a.L * a.tiles_m * a.tiles_n;
+  const int total = a.L * ((a.tiles_m + a.run - 1) / a.run) * a.tiles_n;
   const dim3 grid(((total + 7) / 8) * 8), block(kThreads);
   // A "n" is k-contiguous (KC), A "t" is m-contiguous (RC);
   // B "n" is n-contiguous (RC), B "t" is k-contiguous (KC).
@@ -136,7 +187,7 @@ static BmmArgs make_args(const float* A, const float* B, float* C, const cmk_gem
   a.L = d->L; a.M = d->M; a.N = d->N; a.K = d->K;
   a.tiles_m = (d->M + 127) / 128;
   a.tiles_n = (d->N + 127) / 128;
-  a.group_m = 4;
+  a.run = 1;
   a.vecA = vec_ok(A, d->lda, d->strideA);
   a.vecB = vec_ok(B, d->ldb, d->strideB);
   return a;
@@ -153,6 +204,9 @@ extern "C" int cmk_bmm_f32(const float* A, const float* B, float* C, const cmk_g
   if (!C || (d->K > 0 && (!A || !B))) return fail(CMK_ERR_INVALID_ARG, "cmk_bmm_f32: null pointer");
   if (int e = check_grid((long long)d->L * ((d->M + 127) / 128) * ((d->N + 127) / 128))) return e;
   BmmArgs a = make_args(A, B, C, d);
+  // longer runs amortise the pipeline fill; keep at least ~4 work-groups per CU
+  const long long tiles = (long long)d->L * a.tiles_m * a.tiles_n;
+  a.run = tiles >= 8192 ? 4 : (tiles >= 4096 ? 2 : 1);
   return hip_status(launch_bmm<false>(a, d->transA, d->transB, (hipStream_t)stream),
                     "cmk_bmm_f32 launch");
 }
