@@ -22,6 +22,16 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 PEAK_HBM_GBS = 8000.0
 
+# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc
+# (FETCH_SIZE, WRITE_SIZE: KiB per dispatch).  On this box FETCH_SIZE reads half
+# of the true bytes of a plain 1 GiB device copy and WRITE_SIZE all of them, so
+# traffic = (2 * FETCH_SIZE + WRITE_SIZE) * 1024.  The counters cannot be read
+# from inside this process; the figures are those of the summaries in profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    "min_bmm_large": (2 * 1.52705e6 + 2048) * 1024,      # profiles/min_kernel_min_bmm_large.txt
+    "topk_bmm": (2 * 575644 + 1.57286e6) * 1024,          # profiles/topk_kernel_topk_bmm.txt
+}
+
 
 def make_workloads(torch, cmk, dev):
     """name -> dict(make=..., run=..., flop=..., desc=..., cpu=...)."""
@@ -198,7 +208,7 @@ def main():
         "config": {"workload": wl["desc"], "name": a.workload},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                     "traffic": None, "kernel_ms": round(kern_ms, 4)},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload), "kernel_ms": round(kern_ms, 4)},
     }
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, wl, args)
