@@ -76,22 +76,23 @@ struct TileLayout<RC, T, KS> {
 };
 
 // ---- global -> registers ---------------------------------------------------
-// Each thread fetches NV = T*KS/1024 groups of four consecutive floats.  For
+// Each of the NT threads fetches NV = T*KS/(4*NT) groups of four consecutive floats.  For
 // both kinds the element a thread fetches in pass p sits at
 //     tile + (t / TPR + p * RPP) * ld + (t % TPR) * 4
 // (KC: row-major rows x k, RC: k-major k x rows), so the per-lane part
 // `lane_off` is fixed for a whole kernel and everything else is scalar.
-template <int KIND, int T, int KS>
+template <int KIND, int T, int KS, int NT>
 struct LoadMap {
-  static constexpr int NV = T * KS / 1024;
+  static constexpr int NV = T * KS / (NT * 4);             // float4 per thread
   static constexpr int TPR = KIND == KC ? KS / 4 : T / 4;  // threads per contiguous run
-  static constexpr int RPP = kThreads / TPR;               // runs per pass
+  static constexpr int RPP = NT / TPR;                     // runs per pass
+  static_assert(NV >= 1 && NV * NT * 4 == T * KS, "tile does not divide among the threads");
 };
 
-template <int KIND, int T, int KS>
+template <int KIND, int T, int KS, int NT>
 __device__ __forceinline__ void lane_offsets_bytes(const Operand& o,
-                                                   unsigned (&off)[T * KS / 1024]) {
-  using M = LoadMap<KIND, T, KS>;
+                                                   unsigned (&off)[T * KS / (NT * 4)]) {
+  using M = LoadMap<KIND, T, KS, NT>;
   const int t = threadIdx.x;
 #pragma unroll
   for (int p = 0; p < M::NV; ++p)
@@ -100,10 +101,11 @@ __device__ __forceinline__ void lane_offsets_bytes(const Operand& o,
 
 // r0, k0, K are wave-uniform.  A tile that lies completely inside the matrix
 // takes the branch-free path.
-template <int KIND, int T, int KS>
-__device__ __forceinline__ void gload(const Operand& o, const unsigned (&lane_off)[T * KS / 1024],
-                                      int r0, int k0, int K, f32x4 (&v)[T * KS / 1024]) {
-  using M = LoadMap<KIND, T, KS>;
+template <int KIND, int T, int KS, int NT>
+__device__ __forceinline__ void gload(const Operand& o,
+                                      const unsigned (&lane_off)[T * KS / (NT * 4)], int r0, int k0,
+                                      int K, f32x4 (&v)[T * KS / (NT * 4)]) {
+  using M = LoadMap<KIND, T, KS, NT>;
   constexpr int NV = M::NV, TPR = M::TPR, RPP = M::RPP;
   const int t = threadIdx.x;
   const bool interior = o.vec && (k0 + KS <= K) && (r0 + T <= o.rows) &&
@@ -156,9 +158,9 @@ __device__ __forceinline__ void gload(const Operand& o, const unsigned (&lane_of
 }
 
 // ---- registers -> LDS --------------------------------------------------------
-template <int KIND, int T, int KS>
-__device__ __forceinline__ void lstore(float* lds, const f32x4 (&v)[T * KS / 1024]) {
-  using M = LoadMap<KIND, T, KS>;
+template <int KIND, int T, int KS, int NT>
+__device__ __forceinline__ void lstore(float* lds, const f32x4 (&v)[T * KS / (NT * 4)]) {
+  using M = LoadMap<KIND, T, KS, NT>;
   const int t = threadIdx.x;
   constexpr int pitch = TileLayout<KIND, T, KS>::pitch;
 #pragma unroll
@@ -184,7 +186,7 @@ __device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg, int hal
   }
 }
 
-// Work-group level tile engine.  WX x WY waves (WX*WY == 4), each wave owns
+// Work-group level tile engine.  WX x WY waves (4 or 8 of them), each wave owns
 // BX x BY blocks of 32x32; KS is the contraction depth of one LDS slab.
 //
 // The engine walks a flat sequence of slabs: `ntiles` consecutive X tiles
@@ -196,42 +198,42 @@ __device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg, int hal
 // so the matrix pipe keeps running across slab and tile boundaries.
 template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32>
 struct Core {
-  static_assert(WX * WY == 4, "four waves per work-group");
+  static_assert(WX * WY == 4 || WX * WY == 8, "four or eight waves per work-group");
+  static constexpr int NT = WX * WY * 64;      // threads per work-group
   static constexpr int KS = KS_;
   static constexpr int NG = KS / 8;            // k-groups per slab
   static constexpr int WRITE_AT = NG / 2 - 1;  // k-group after which the next slab goes to LDS
   static constexpr int TX = WX * BX * 32;
   static constexpr int TY = WY * BY * 32;
-  static_assert(NG >= 2 && NG % 2 == 0 && (TX * KS) % 1024 == 0 && (TY * KS) % 1024 == 0,
-                "tile shape");
+  static_assert(NG >= 2 && NG % 2 == 0, "slab depth");
   static constexpr int xFloats = TileLayout<XK, TX, KS>::floats;
   static constexpr int yFloats = TileLayout<YK, TY, KS>::floats;
   static constexpr int bufFloats = xFloats + yFloats;
   static constexpr int ldsFloats = 2 * bufFloats;
 
-  f32x4 xv[TX * KS / 1024];  // slab in flight from global memory
-  f32x4 yv[TY * KS / 1024];
+  f32x4 xv[TX * KS / (NT * 4)];  // slab in flight from global memory
+  f32x4 yv[TY * KS / (NT * 4)];
   f32x4 xf[2][BX];           // fragments; [0] holds k-group 0 of the current slab at slab entry
   f32x4 yf[2][BY];
   int it, iters, S;          // flat slab counter (wave-uniform)
   int lt, ls;                // (tile, slab) of the next slab to fetch (wave-uniform)
   int xbase, y0, K;
   int xr, yr, half;
-  unsigned xoff[TX * KS / 1024];  // this lane's byte offsets inside an operand tile
-  unsigned yoff[TY * KS / 1024];
+  unsigned xoff[TX * KS / (NT * 4)];  // this lane's byte offsets inside an operand tile
+  unsigned yoff[TY * KS / (NT * 4)];
 
   __device__ __forceinline__ void load(const Operand& X, const Operand& Y) {
     // the slab coordinates are the same for every lane; saying so keeps the
     // address arithmetic on the scalar unit
     const int x0 = __builtin_amdgcn_readfirstlane(xbase + lt * TX);
     const int k0 = __builtin_amdgcn_readfirstlane(ls * KS);
-    gload<XK, TX, KS>(X, xoff, x0, k0, K, xv);
-    gload<YK, TY, KS>(Y, yoff, y0, k0, K, yv);
+    gload<XK, TX, KS, NT>(X, xoff, x0, k0, K, xv);
+    gload<YK, TY, KS, NT>(Y, yoff, y0, k0, K, yv);
     if (++ls == S) { ls = 0; ++lt; }
   }
   __device__ __forceinline__ void store(float* buf) {
-    lstore<XK, TX, KS>(buf, xv);
-    lstore<YK, TY, KS>(buf + xFloats, yv);
+    lstore<XK, TX, KS, NT>(buf, xv);
+    lstore<YK, TY, KS, NT>(buf + xFloats, yv);
   }
   __device__ __forceinline__ void read_frags(const float* buf, int kg, f32x4 (&fx)[BX],
                                              f32x4 (&fy)[BY]) {
@@ -255,8 +257,8 @@ struct Core {
     K = __builtin_amdgcn_readfirstlane(K_);
     S = max(1, (K + KS - 1) / KS);
     iters = __builtin_amdgcn_readfirstlane(ntiles) * S;
-    lane_offsets_bytes<XK, TX, KS>(X, xoff);
-    lane_offsets_bytes<YK, TY, KS>(Y, yoff);
+    lane_offsets_bytes<XK, TX, KS, NT>(X, xoff);
+    lane_offsets_bytes<YK, TY, KS, NT>(Y, yoff);
     it = 0;
     lt = 0;
     ls = 0;

@@ -1,16 +1,16 @@
 // topk_bmm: fused per-row top-128 (largest, sorted descending) of A@B along
 // one axis; the product never reaches HBM.
 //
-// X = the reduced axis (inside a lane), Y = the kept axis.  A work-group owns a
-// strip of 32 complete output rows and walks the reduced axis in chunks of
-// 1024 candidates (8 tiles of 128) whose accumulators all stay in registers.
-// After each chunk the accumulators go through LDS, eight rows at a time, so
-// that one wave sees one row's 1024 candidates (16 per lane) together with the
-// row's running list (2 per lane); select128() keeps the best 128 in the
-// running list in LDS.  After the last chunk each wave orders its rows' lists
-// with the bitonic network and stores them.  When the kept axis has too few
-// strips to fill the chip, the reduced axis is cut into `splits` ranges whose
-// unordered lists go to a workspace and are merged by a second kernel.
+// X = the reduced axis (inside a lane), Y = the kept axis.  A work-group of
+// eight waves owns a strip of 64 complete output rows and walks the reduced
+// axis in chunks of 1024 candidates (8 tiles of 128) whose accumulators all
+// stay in registers.  After each chunk the accumulators go through LDS, sixteen
+// rows at a time, so that one wave sees one row's 1024 candidates (16 per lane)
+// together with the row's running list (2 per lane); select128() keeps the best
+// 128 in the running list in LDS.  After the last chunk each wave orders its
+// rows' lists with the bitonic network and stores them.  When the kept axis has
+// too few strips to fill the chip, the reduced axis is cut into `splits` ranges
+// whose unordered lists go to a workspace and are merged by a second kernel.
 //
 // Plays the role of topk_bmm_* with topk_dim_1 / topk_dim_2, bitonic_sort_128,
 // bitonic_sort_256 and the row mutex (reference kernels/topkbmm.cu:13-303,
@@ -35,24 +35,41 @@ struct TopkArgs {
   int ystrips, xtiles, splits, tiles_per_split;
 };
 
-template <int XK, int YK>
-__global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
-  using C = Core<XK, YK, 4, 1, 1, 1>;
-  static_assert(C::TX == 128 && C::TY == 32, "tile shape");
-  constexpr int opFloats = C::ldsFloats;
-  static_assert(opFloats >= 8 * kStagePitch + 4 * 2 * kTop,
-                "staging area and band lists alias the operand buffers");
-  __shared__ __attribute__((aligned(16))) float lds[opFloats];
-  __shared__ entry_t list[32][kTop];   // running top-128 of every row of the strip
+constexpr int kTopkThreads = 512;
+constexpr int kStripRows = 64;    // output rows per work-group
+constexpr int kPassRows = 16;     // rows staged through LDS per selection pass
 
-  const int total = a.L * a.ystrips * a.splits;
-  const int logical = xcd_logical_id(blockIdx.x, total);
+// MULTI = false: the whole reduced axis is one chunk (at most 1024 candidates).
+// The running lists are then only written after the product is finished, so
+// they may share LDS with the operand buffers, which leaves room for slabs of
+// depth 64 (half as many barriers per MFMA).  MULTI = true keeps the lists
+// apart and uses slabs of depth 32.
+template <int XK, int YK, bool MULTI>
+__global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
+  // eight waves: wave % 4 picks 32 of a tile's 128 candidates, wave / 4 one of
+  // the two 32-row halves of the strip.  One work-group per CU; its two waves
+  // per SIMD are always in the same phase, because on this part a wave's
+  // selection (VALU) work does not hide behind another wave's MFMA stream.
+  using C = Core<XK, YK, 4, 2, 1, 1, MULTI ? 32 : 64>;
+  static_assert(C::TX == 128 && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
+  constexpr int stageFloats = kPassRows * kStagePitch;
+  constexpr int bandFloats = 8 * kTop * 2;  // one 128-entry band list per wave
+  constexpr int listFloats = kStripRows * kTop * 2;
+  constexpr int selFloats = stageFloats + bandFloats + listFloats;
+  static_assert(C::ldsFloats <= (MULTI ? stageFloats + bandFloats : selFloats),
+                "operand buffers must not reach the lists when these carry state between chunks");
+  __shared__ __attribute__((aligned(16))) float lds[selFloats];
+  // running top-128 of every row of the strip
+  entry_t(*list)[kTop] = reinterpret_cast<entry_t(*)[kTop]>(lds + stageFloats + bandFloats);
+
+  const int per_split = a.L * a.ystrips;
+  const int logical = xcd_logical_id(blockIdx.x, per_split * a.splits);
   if (logical < 0) return;
-  const int split = logical / (a.L * a.ystrips);
-  const int rem = logical - split * (a.L * a.ystrips);
+  const int split = logical / per_split;
+  const int rem = logical - split * per_split;
   const int b = rem / a.ystrips;
   const int ystrip = rem - b * a.ystrips;
-  const int y0 = ystrip * C::TY;
+  const int y0 = ystrip * kStripRows;
   const int xt_begin = split * a.tiles_per_split;
   const int xt_end = min(a.xtiles, xt_begin + a.tiles_per_split);
 
@@ -66,11 +83,15 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
   const int wave = threadIdx.x >> 6;
   const int l32 = lane & 31;
   const int half = lane >> 5;
+  const int wx = wave & 3;   // which 32 candidates of a tile
+  const int wy = wave >> 2;  // which half of the strip's rows
 
-  // running lists start empty
-  for (int e = threadIdx.x; e < 32 * kTop; e += kThreads) (&list[0][0])[e] = 0ull;
-  __syncthreads();
-  entry_t* band = reinterpret_cast<entry_t*>(lds + 8 * kStagePitch) + wave * kTop;
+  if constexpr (MULTI) {
+    // running lists start empty
+    for (int e = threadIdx.x; e < kStripRows * kTop; e += kTopkThreads) (&list[0][0])[e] = 0ull;
+    __syncthreads();
+  }
+  entry_t* band = reinterpret_cast<entry_t*>(lds + stageFloats) + wave * kTop;
   uint32_t seed[1] = {0u};
 
   C core;
@@ -88,13 +109,14 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
     }
     __syncthreads();  // all fragment reads are done; the buffers become the staging area
 
-    // selection, eight rows of the strip per pass
+    // selection, sixteen rows of the strip per pass
     const int xc0 = xt0 * C::TX;
 #pragma unroll 1
-    for (int g = 0; g < 4; ++g) {
+    for (int g = 0; g < kStripRows / kPassRows; ++g) {
       if (g) __syncthreads();  // previous pass has been read
-      if ((l32 >> 3) == g) {
-        float* row = lds + (l32 & 7) * kStagePitch + wave * 32 + 4 * half;
+      // rows 16g .. 16g+15 live in the waves with wy == g / 2, lanes l32 / 16 == g % 2
+      if (wy == (g >> 1) && (l32 >> 4) == (g & 1)) {
+        float* row = lds + (l32 & 15) * kStagePitch + wx * 32 + 4 * half;
 #pragma unroll
         for (int i = 0; i < kChunkTiles; ++i)
 #pragma unroll
@@ -107,17 +129,18 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
       __syncthreads();
 #pragma unroll 1
       for (int rr = 0; rr < 2; ++rr) {
-        const int r = 8 * g + 2 * wave + rr;  // row of the strip, owned by this wave
+        const int pr = 2 * wave + rr;          // row of the pass, owned by this wave
+        const int r = kPassRows * g + pr;      // row of the strip
         if (y0 + r >= Yext) continue;
         entry_t* const outs[1] = {list[r]};
         entry_t* const bands[1] = {band};
-        const float* src = lds + (r & 7) * kStagePitch;
+        const float* src = lds + pr * kStagePitch;
         const int xl = xc0 + lane;
         uint32_t key[1][18];
 #pragma unroll
         for (int j = 0; j < 16; ++j)
           key[0][j] = xl + 64 * j < x_limit ? f2key(src[lane + 64 * j]) : 0u;
-        if (xt0 == xt_begin) {
+        if (!MULTI || xt0 == xt_begin) {
           // first chunk: the running list is empty
           uint32_t k16[1][16];
 #pragma unroll
@@ -137,8 +160,8 @@ __global__ __launch_bounds__(kThreads, 2) void topk_kernel(TopkArgs a) {
 
   // each wave finishes the rows it owns, two at a time
 #pragma unroll 1
-  for (int g = 0; g < 4; ++g) {
-    const int r0 = 8 * g + 2 * wave;
+  for (int g = 0; g < kStripRows / kPassRows; ++g) {
+    const int r0 = kPassRows * g + 2 * wave;
     if (a.splits == 1) {
       const entry_t* const lists[2] = {list[r0], list[r0 + 1]};
       float* vals[2];
@@ -246,12 +269,12 @@ __global__ __launch_bounds__(kThreads) void topk1d_partial_kernel(const float* a
 
 static void plan_topk(int L, int Xext, int Yext, int* ystrips, int* xtiles, int* splits,
                       int* tiles_per_split) {
-  *ystrips = ceil_div(Yext, 32);
+  *ystrips = ceil_div(Yext, kStripRows);
   *xtiles = ceil_div(Xext, 128);
   const long long strips = (long long)L * *ystrips;
   const int chunks = ceil_div(*xtiles, kChunkTiles);
   int want = 1;
-  if (strips < 512) want = (int)((512 + strips - 1) / strips);
+  if (strips < 256) want = (int)((256 + strips - 1) / strips);
   if (want > chunks) want = chunks;
   if (want < 1) want = 1;
   const int chunks_per_split = ceil_div(chunks, want);
@@ -326,17 +349,24 @@ extern "C" int cmk_topk_bmm_f32(const float* A, const float* B, float* values, l
   }
   const long long total = (long long)d->L * a.ystrips * a.splits;
   if (int e = check_grid(total)) return e;
-  const dim3 grid((unsigned)(((total + 7) / 8) * 8)), block(kThreads);
+  const dim3 grid((unsigned)(((total + 7) / 8) * 8)), block(kTopkThreads);
   hipStream_t st = (hipStream_t)stream;
-  if (xk == KC && yk == KC) hipLaunchKernelGGL((topk_kernel<KC, KC>), grid, block, 0, st, a);
-  else if (xk == KC && yk == RC) hipLaunchKernelGGL((topk_kernel<KC, RC>), grid, block, 0, st, a);
-  else if (xk == RC && yk == KC) hipLaunchKernelGGL((topk_kernel<RC, KC>), grid, block, 0, st, a);
-  else hipLaunchKernelGGL((topk_kernel<RC, RC>), grid, block, 0, st, a);
+  const bool multi = a.splits > 1 || a.xtiles > kChunkTiles;
+#define CMK_TOPK_LAUNCH(XKIND, YKIND)                                                      \
+  do {                                                                                     \
+    if (multi) hipLaunchKernelGGL((topk_kernel<XKIND, YKIND, true>), grid, block, 0, st, a); \
+    else hipLaunchKernelGGL((topk_kernel<XKIND, YKIND, false>), grid, block, 0, st, a);     \
+  } while (0)
+  if (xk == KC && yk == KC) CMK_TOPK_LAUNCH(KC, KC);
+  else if (xk == KC && yk == RC) CMK_TOPK_LAUNCH(KC, RC);
+  else if (xk == RC && yk == KC) CMK_TOPK_LAUNCH(RC, KC);
+  else CMK_TOPK_LAUNCH(RC, RC);
+#undef CMK_TOPK_LAUNCH
   if (int e = hip_status(hipGetLastError(), "cmk_topk_bmm_f32 launch")) return e;
   if (a.splits > 1) {
     const long long rows = (long long)d->L * Yext;
     if (int e = check_grid((rows + 3) / 4)) return e;
-    hipLaunchKernelGGL(topk_merge_kernel, dim3((unsigned)((rows + 3) / 4)), block, 0, st,
+    hipLaunchKernelGGL(topk_merge_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(kThreads), 0, st,
                        a.part, values, indices, rows, a.splits, k);
     if (int e = hip_status(hipGetLastError(), "cmk_topk_bmm_f32 merge launch")) return e;
   }
