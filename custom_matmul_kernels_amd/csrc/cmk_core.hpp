@@ -192,10 +192,12 @@ __device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg, int hal
 // The engine walks a flat sequence of slabs: `ntiles` consecutive X tiles
 // (starting at element `xbase`) against one Y strip, S = ceil(K/KS) slabs per
 // tile.  While slab i is multiplied, slab i+1 is written to the other LDS
-// buffer (in the middle of the slab, so the writes hide behind MFMAs) and slab
-// i+2 is on its way from global memory.  The one barrier per slab sits before
-// the last k-group; right after it the first fragments of slab i+1 are read,
-// so the matrix pipe keeps running across slab and tile boundaries.
+// buffer (in the middle of the slab) and slab i+2 is on its way from global
+// memory.  The one barrier per slab sits inside the last k-group; right after
+// it the first fragments of slab i+1 are read, so the matrix pipe keeps running
+// across slab and tile boundaries.  Inside a k-group all LDS and global traffic
+// is issued directly behind the group's first MFMA step, where it costs no
+// matrix-pipe time.
 template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32>
 struct Core {
   static_assert(WX * WY == 4 || WX * WY == 8, "four or eight waves per work-group");
@@ -279,15 +281,28 @@ struct Core {
       const bool has2 = it + 2 < iters;
 #pragma unroll
       for (int kg = 0; kg < NG; ++kg) {
+        // first k-step of the group; everything that is not an MFMA is issued
+        // right behind it, in the shadow of the matrix pipe
+#pragma unroll
+        for (int bx = 0; bx < BX; ++bx)
+#pragma unroll
+          for (int by = 0; by < BY; ++by)
+            acc[bx][by] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                xf[kg & 1][bx][0], yf[kg & 1][by][0], acc[bx][by], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
         if (kg + 1 < NG) {
           read_frags(cur, kg + 1, xf[(kg + 1) & 1], yf[(kg + 1) & 1]);
         } else if (has1) {
           __syncthreads();
           read_frags(nxt, 0, xf[0], yf[0]);
         }
-        __builtin_amdgcn_sched_barrier(0);  // LDS reads stay above the MFMAs they overlap with
+        if (kg == WRITE_AT) {
+          if (has1) store(nxt);
+          if (has2) load(X, Y);
+        }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 1; j < 4; ++j)
 #pragma unroll
           for (int bx = 0; bx < BX; ++bx)
 #pragma unroll
@@ -295,10 +310,6 @@ struct Core {
               acc[bx][by] = __builtin_amdgcn_mfma_f32_32x32x2f32(
                   xf[kg & 1][bx][j], yf[kg & 1][by][j], acc[bx][by], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (kg == WRITE_AT) {
-          if (has1) store(nxt);
-          if (has2) load(X, Y);
-        }
       }
       ++it;
     }
