@@ -47,6 +47,19 @@ int check_grid(long long work_groups) {
   return CMK_OK;
 }
 
+int compute_units() {
+  static thread_local int cached_dev = -1, cached_cus = 256;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (dev != cached_dev) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
+      cached_cus = cus;
+    cached_dev = dev;
+  }
+  return cached_cus;
+}
+
 size_t min_workspace_bytes(int L, int Xext, int Yext, int K);
 size_t topk_workspace_bytes(int L, int Xext, int Yext);
 size_t topk1d_workspace_bytes(long long n);

@@ -26,4 +26,7 @@ static inline int vec_ok(const void* p, long long ld, long long stride) {
 
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Compute units of the current device (cached per device).
+int compute_units();
+
 }  // namespace cmk

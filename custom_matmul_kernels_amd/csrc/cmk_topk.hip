@@ -62,9 +62,27 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   // running top-128 of every row of the strip
   entry_t(*list)[kTop] = reinterpret_cast<entry_t(*)[kTop]>(lds + stageFloats + bandFloats);
 
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int l32 = lane & 31;
+  const int half = lane >> 5;
+  const int wx = wave & 3;   // which 32 candidates of a tile
+  const int wy = wave >> 2;  // which half of the strip's rows
+  entry_t* band = reinterpret_cast<entry_t*>(lds + stageFloats) + wave * kTop;
+  // the previous row's threshold seeds the next search; it carries over from
+  // strip to strip, since neighbouring strips are statistically alike
+  uint32_t seed[1] = {0u};
+
+  // A work-group walks strips blockIdx.x, blockIdx.x + gridDim.x, ... (the
+  // grid is sized to the machine, not to the problem).
   const int per_split = a.L * a.ystrips;
-  const int logical = xcd_logical_id(blockIdx.x, per_split * a.splits);
-  if (logical < 0) return;
+  const int total = per_split * a.splits;
+  const int padded = ((total + 7) >> 3) << 3;
+#pragma unroll 1
+  for (int hw = blockIdx.x; hw < padded; hw += gridDim.x) {
+  const int logical = xcd_logical_id(hw, total);
+  if (logical < 0) continue;
+  __syncthreads();  // the previous strip's lists have been stored
   const int split = logical / per_split;
   const int rem = logical - split * per_split;
   const int b = rem / a.ystrips;
@@ -79,21 +97,11 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   const int x_limit = min(X.rows, xt_end * C::TX);
   const int Yext = Y.rows;
 
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int l32 = lane & 31;
-  const int half = lane >> 5;
-  const int wx = wave & 3;   // which 32 candidates of a tile
-  const int wy = wave >> 2;  // which half of the strip's rows
-
   if constexpr (MULTI) {
     // running lists start empty
     for (int e = threadIdx.x; e < kStripRows * kTop; e += kTopkThreads) (&list[0][0])[e] = 0ull;
     __syncthreads();
   }
-  entry_t* band = reinterpret_cast<entry_t*>(lds + stageFloats) + wave * kTop;
-  uint32_t seed[1] = {0u};
-
   C core;
 
   for (int xt0 = xt_begin; xt0 < xt_end; xt0 += kChunkTiles) {
@@ -187,6 +195,7 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
       }
     }
   }
+  }  // strips
 }
 
 // One wave per output row: folds `parts` unordered 128-entry lists into one,
@@ -349,7 +358,10 @@ extern "C" int cmk_topk_bmm_f32(const float* A, const float* B, float* values, l
   }
   const long long total = (long long)d->L * a.ystrips * a.splits;
   if (int e = check_grid(total)) return e;
-  const dim3 grid((unsigned)(((total + 7) / 8) * 8)), block(kTopkThreads);
+  // one eight-wave work-group per CU is resident at a time; two per CU even out the tail
+  const long long padded = ((total + 7) / 8) * 8;
+  const long long machine = 2ll * compute_units();
+  const dim3 grid((unsigned)(padded < machine ? padded : machine)), block(kTopkThreads);
   hipStream_t st = (hipStream_t)stream;
   const bool multi = a.splits > 1 || a.xtiles > kChunkTiles;
 #define CMK_TOPK_LAUNCH(XKIND, YKIND)                                                      \
