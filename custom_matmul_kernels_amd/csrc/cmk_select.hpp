@@ -6,12 +6,11 @@
 //   1. Bracket the key of the 128th largest, [lo, hi), by counting candidates
 //      >= t with wave ballots.  The bracket starts around the previous row's
 //      answer (rows of one strip are statistically alike) and is bisected until
-//      it holds at most 128 candidates.
-//   2. One pass over the registers sends every candidate >= hi to the output
-//      list and every candidate inside the bracket to a band list (both in LDS,
-//      as 64-bit (key, ~index) entries).
-//   3. The band, now two entries per lane, is bisected to the exact threshold
-//      and its winners are appended to the output list.
+//      at most 256 candidates lie at or above lo.
+//   2. One pass over the registers compacts those candidates into a list in
+//      LDS, as 64-bit (key, ~index) entries.
+//   3. The list, now four entries per lane, is bisected to the exact threshold
+//      and the 128 winners are written to the output list.
 // The output list is unordered; bitonic128_desc() orders it once, at the very
 // end, so that values descend and equal values come out by ascending index.
 //
@@ -60,159 +59,121 @@ __device__ __forceinline__ uint32_t bracket_mid(uint32_t lo, uint32_t hi) {
   return (lo == 0 && hi == 0) ? 0x80000000u : lo + ((hi - lo) >> 1);
 }
 
-// Selects, for each of R rows at once, the 128 largest keys among key[r][0..NR)
-// of all 64 lanes and writes them as entries to out[r][0..128) (LDS owned by
-// this wave).  The R rows are independent; working on them side by side lets
-// the counting chains of one row hide the latency of the other.  band[r] is 128
-// entries of wave-private LDS scratch.  seed[r] carries the threshold key from
-// one call to the next (0 = none); idx_of(r, j) is the index of candidate
-// key[r][j] of this lane.  Ties at the threshold: earliest (register,
-// lane) position first.  Fewer than 128 real candidates leave empty entries.
-template <int NR, int R, class IdxOf>
-__device__ __forceinline__ void select128(const uint32_t (&key)[R][NR], IdxOf&& idx_of,
-                                          uint32_t (&seed)[R], entry_t* const (&band)[R],
-                                          entry_t* const (&out)[R]) {
-  const int lane = threadIdx.x & 63;
-  // bracket: count(>= lo) >= 128 > count(>= hi); hi == 0 stands for 2^32
-  uint32_t lo[R], hi[R];
-  int c_lo[R], c_hi[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) { lo[r] = 0; hi[r] = 0; c_lo[r] = NR * 64; c_hi[r] = 0; }
+constexpr int kCand = 256;  // capacity of the candidate list select128() works in
 
-  auto count_ge = [&](int r, uint32_t t) {
+// Selects the 128 largest keys among key[0..NR) of all 64 lanes and writes them
+// as entries to out[0..128) (LDS owned by this wave).  `cand` is kCand entries of
+// wave-private LDS scratch.  `seed` carries the threshold key from one call to
+// the next (0 = none); idx_of(j) is the index of candidate key[j] of this lane.
+// Ties at the threshold: earliest (register, lane) position first.  Fewer than
+// 128 real candidates leave empty entries.
+template <int NR, class IdxOf>
+__device__ __forceinline__ void select128(const uint32_t (&key)[NR], IdxOf&& idx_of,
+                                          uint32_t& seed, entry_t* cand, entry_t* out) {
+  const int lane = threadIdx.x & 63;
+  auto count_ge = [&](uint32_t t) {
     int c = 0;
 #pragma unroll
-    for (int j = 0; j < NR; ++j) c += __popcll(__ballot(key[r][j] >= t));
+    for (int j = 0; j < NR; ++j) c += __popcll(__ballot(key[j] >= t));
     return c;
   };
-  auto narrow = [&](int r, uint32_t t, int c) {
-    if (c >= kTop) { lo[r] = t; c_lo[r] = c; } else { hi[r] = t; c_hi[r] = c; }
-  };
-
-  constexpr uint32_t D = 1u << 20;  // +-12% of a float's magnitude
-  {
-    uint32_t t[R];
-    int c[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) t[r] = seed[r] > D ? seed[r] - D : 1u;
-#pragma unroll
-    for (int r = 0; r < R; ++r) c[r] = seed[r] ? count_ge(r, t[r]) : 0;
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-      if (seed[r]) narrow(r, t[r], c[r]);
-    bool second[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      second[r] = seed[r] && hi[r] == 0 && seed[r] < 0xFFFFFFFFu - D;
-      t[r] = seed[r] + D;
+  // bracket: count(>= lo) >= 128 > count(>= hi); hi == 0 stands for 2^32
+  uint32_t lo = 0, hi = 0;
+  int c_lo = NR * 64, c_hi = 0;
+  if (seed) {
+    constexpr uint32_t D = 1u << 20;  // +-12% of a float's magnitude
+    const uint32_t t0 = seed > D ? seed - D : 1u;
+    const int c0 = count_ge(t0);
+    if (c0 >= kTop) { lo = t0; c_lo = c0; } else { hi = t0; c_hi = c0; }
+    if (hi == 0 && seed < 0xFFFFFFFFu - D) {
+      const uint32_t t1 = seed + D;
+      const int c1 = count_ge(t1);
+      if (c1 >= kTop) { lo = t1; c_lo = c1; } else { hi = t1; c_hi = c1; }
     }
-#pragma unroll
-    for (int r = 0; r < R; ++r) c[r] = second[r] ? count_ge(r, t[r]) : 0;
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-      if (second[r]) narrow(r, t[r], c[r]);
   }
-  for (;;) {
-    bool act[R], any = false;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      act[r] = c_lo[r] - c_hi[r] > kTop && hi[r] - lo[r] != 1u;
-      any = any || act[r];
-    }
-    if (!any) break;
-    uint32_t t[R];
-    int c[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) t[r] = bracket_mid(lo[r], hi[r]);
-#pragma unroll
-    for (int r = 0; r < R; ++r) c[r] = act[r] ? count_ge(r, t[r]) : 0;
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-      if (act[r]) narrow(r, t[r], c[r]);
+  while (c_lo > kCand && hi - lo != 1u) {
+    const uint32_t mid = bracket_mid(lo, hi);
+    const int c = count_ge(mid);
+    if (c >= kTop) { lo = mid; c_lo = c; } else { hi = mid; c_hi = c; }
   }
 
-  // one pass: candidates >= hi go to out[0, c_hi), candidates in [lo, hi) to the band
-  int base_band[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    int base_out = 0;
-    base_band[r] = 0;
+  if (c_lo <= kCand) {
+    // one pass: every candidate >= lo goes to the candidate list, in (register,
+    // lane) order; there are at least 128 and at most 256 of them
+    int base = 0;
 #pragma unroll
     for (int j = 0; j < NR; ++j) {
-      const uint32_t k = key[r][j];
-      const bool ge_lo = k >= lo[r];
-      const bool ge_hi = hi[r] != 0 && k >= hi[r];
-      const unsigned long long m_lo = __ballot(ge_lo);
-      const unsigned long long m_hi = __ballot(ge_hi);
-      const unsigned long long m_band = m_lo & ~m_hi;
-      const entry_t e = pack_entry(k, k ? idx_of(r, j) : -1);
-      if (ge_hi) {
-        out[r][base_out + prefix_in(m_hi)] = e;
-      } else if (ge_lo) {
-        const int pos = base_band[r] + prefix_in(m_band);
-        if (pos < kTop) band[r][pos] = e;
-      }
-      base_out += __popcll(m_hi);
-      base_band[r] += __popcll(m_band);
+      const bool ge = key[j] >= lo;
+      const unsigned long long m = __ballot(ge);
+      const int pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m >> 32),
+                                                __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m), base));
+      if (ge) cand[pos] = pack_entry(key[j], idx_of(j));
+      base += __popcll(m);
     }
-  }
-
-  // the band: two entries per lane and row, `need` of them are wanted
-  int need[R], cb_lo[R];
-  entry_t b0[R], b1[R];
-  uint32_t k0[R], k1[R];
-  bool v0[R], v1[R];
+    // four entries per lane; bisect to the exact threshold: the largest t with
+    // count(>= t) >= 128, stopping early when the count is exactly 128
+    entry_t e[4];
+    uint32_t k[4];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    need[r] = kTop - c_hi[r];
-    const int nband = base_band[r] < kTop ? base_band[r] : kTop;
-    v0[r] = lane < nband;
-    v1[r] = lane + 64 < nband;
-    b0[r] = v0[r] ? band[r][lane] : 0ull;
-    b1[r] = v1[r] ? band[r][lane + 64] : 0ull;
-    k0[r] = entry_key(b0[r]);
-    k1[r] = entry_key(b1[r]);
-    cb_lo[r] = base_band[r];  // everything in the band is >= lo
-  }
-  // exact threshold inside the band: largest t with count(band >= t) >= need
-  for (;;) {
-    bool act[R], any = false;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      act[r] = cb_lo[r] != need[r] && hi[r] - lo[r] != 1u;
-      any = any || act[r];
+    for (int m = 0; m < 4; ++m) {
+      const bool valid = lane + 64 * m < c_lo;
+      e[m] = valid ? cand[lane + 64 * m] : 0ull;
+      k[m] = entry_key(e[m]);
+      if (k[m] == 0u) e[m] = 0ull;  // "no candidate" carries index -1
     }
-    if (!any) break;
+    int n_lo = c_lo;
+    while (n_lo != kTop && hi - lo != 1u) {
+      const uint32_t mid = bracket_mid(lo, hi);
+      int c = 0;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const uint32_t mid = bracket_mid(lo[r], hi[r]);
-      const int c = __popcll(__ballot(v0[r] && k0[r] >= mid)) + __popcll(__ballot(v1[r] && k1[r] >= mid));
-      if (act[r]) {
-        if (c >= need[r]) { lo[r] = mid; cb_lo[r] = c; } else { hi[r] = mid; }
-      }
+      for (int m = 0; m < 4; ++m) c += __popcll(__ballot(lane + 64 * m < c_lo && k[m] >= mid));
+      if (c >= kTop) { lo = mid; n_lo = c; } else { hi = mid; }
     }
-  }
-  // winners: every band entry >= lo when that is exactly `need` of them,
-  // otherwise (ties at lo) those above lo and then the first ones equal to lo
+    // winners: all entries >= lo if that is exactly 128, otherwise (ties at lo)
+    // those above lo and then the first ones equal to lo
+    const bool exact = n_lo == kTop;
+    int pos_gt = 0;
+    unsigned long long mg[4];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const bool exact = cb_lo[r] == need[r];
-    const bool g0 = v0[r] && (exact ? k0[r] >= lo[r] : k0[r] > lo[r]);
-    const bool g1 = v1[r] && (exact ? k1[r] >= lo[r] : k1[r] > lo[r]);
-    const unsigned long long mg0 = __ballot(g0), mg1 = __ballot(g1);
-    const int ng0 = __popcll(mg0), ng = ng0 + __popcll(mg1);
-    if (g0) out[r][c_hi[r] + prefix_in(mg0)] = b0[r];
-    if (g1) out[r][c_hi[r] + ng0 + prefix_in(mg1)] = b1[r];
+    for (int m = 0; m < 4; ++m) {
+      const bool valid = lane + 64 * m < c_lo;
+      const bool g = valid && (exact ? k[m] >= lo : k[m] > lo);
+      mg[m] = __ballot(g);
+      if (g) out[pos_gt + prefix_in(mg[m])] = e[m];
+      pos_gt += __popcll(mg[m]);
+    }
     if (!exact) {
-      const bool q0 = v0[r] && k0[r] == lo[r], q1 = v1[r] && k1[r] == lo[r];
-      const unsigned long long mq0 = __ballot(q0), mq1 = __ballot(q1);
-      const int p0 = c_hi[r] + ng + prefix_in(mq0);
-      const int p1 = c_hi[r] + ng + __popcll(mq0) + prefix_in(mq1);
-      if (q0 && p0 < kTop) out[r][p0] = b0[r];
-      if (q1 && p1 < kTop) out[r][p1] = b1[r];
+      int pos_eq = pos_gt;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const bool q = lane + 64 * m < c_lo && k[m] == lo;
+        const unsigned long long mq = __ballot(q);
+        const int p = pos_eq + prefix_in(mq);
+        if (q && p < kTop) out[p] = e[m];
+        pos_eq += __popcll(mq);
+      }
     }
-    seed[r] = lo[r];
+  } else {
+    // more than 256 candidates share the key lo (hi == lo + 1): take every
+    // candidate above lo, then the first ones equal to lo
+    int base = 0;
+#pragma unroll
+    for (int j = 0; j < NR; ++j) {
+      const bool g = key[j] > lo;
+      const unsigned long long m = __ballot(g);
+      if (g) out[base + prefix_in(m)] = pack_entry(key[j], idx_of(j));
+      base += __popcll(m);
+    }
+#pragma unroll
+    for (int j = 0; j < NR; ++j) {
+      const bool q = key[j] == lo;
+      const unsigned long long m = __ballot(q);
+      const int p = base + prefix_in(m);
+      if (q && p < kTop) out[p] = lo ? pack_entry(lo, idx_of(j)) : 0ull;
+      base += __popcll(m);
+    }
   }
+  seed = lo;
 }
 
 // Value of `v` in lane (lane ^ STRIDE).

@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   using C = Core<XK, YK, 4, 2, 1, 1, MULTI ? 32 : 64>;
   static_assert(C::TX == 128 && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
   constexpr int stageFloats = kPassRows * kStagePitch;
-  constexpr int bandFloats = 8 * kTop * 2;  // one 128-entry band list per wave
+  constexpr int bandFloats = 8 * kCand * 2;  // one candidate list per wave
   constexpr int listFloats = kStripRows * kTop * 2;
   constexpr int selFloats = stageFloats + bandFloats + listFloats;
   static_assert(C::ldsFloats <= (MULTI ? stageFloats + bandFloats : selFloats),
@@ -68,10 +68,10 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   const int half = lane >> 5;
   const int wx = wave & 3;   // which 32 candidates of a tile
   const int wy = wave >> 2;  // which half of the strip's rows
-  entry_t* band = reinterpret_cast<entry_t*>(lds + stageFloats) + wave * kTop;
+  entry_t* cand = reinterpret_cast<entry_t*>(lds + stageFloats) + wave * kCand;
   // the previous row's threshold seeds the next search; it carries over from
   // strip to strip, since neighbouring strips are statistically alike
-  uint32_t seed[1] = {0u};
+  uint32_t seed = 0u;
 
   // A work-group walks strips blockIdx.x, blockIdx.x + gridDim.x, ... (the
   // grid is sized to the machine, not to the problem).
@@ -140,27 +140,30 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
         const int pr = 2 * wave + rr;          // row of the pass, owned by this wave
         const int r = kPassRows * g + pr;      // row of the strip
         if (y0 + r >= Yext) continue;
-        entry_t* const outs[1] = {list[r]};
-        entry_t* const bands[1] = {band};
         const float* src = lds + pr * kStagePitch;
         const int xl = xc0 + lane;
-        uint32_t key[1][18];
+        uint32_t key[18];
+        if (xc0 + 1024 <= x_limit) {
 #pragma unroll
-        for (int j = 0; j < 16; ++j)
-          key[0][j] = xl + 64 * j < x_limit ? f2key(src[lane + 64 * j]) : 0u;
+          for (int j = 0; j < 16; ++j) key[j] = f2key(src[lane + 64 * j]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 16; ++j)
+            key[j] = xl + 64 * j < x_limit ? f2key(src[lane + 64 * j]) : 0u;
+        }
         if (!MULTI || xt0 == xt_begin) {
           // first chunk: the running list is empty
-          uint32_t k16[1][16];
+          uint32_t k16[16];
 #pragma unroll
-          for (int j = 0; j < 16; ++j) k16[0][j] = key[0][j];
-          select128<16, 1>(k16, [&](int, int j) { return xl + 64 * j; }, seed, bands, outs);
+          for (int j = 0; j < 16; ++j) k16[j] = key[j];
+          select128<16>(k16, [&](int j) { return xl + 64 * j; }, seed, cand, list[r]);
         } else {
           const entry_t e0 = list[r][lane], e1 = list[r][lane + 64];
-          key[0][16] = entry_key(e0);
-          key[0][17] = entry_key(e1);
+          key[16] = entry_key(e0);
+          key[17] = entry_key(e1);
           const int ri0 = entry_idx(e0), ri1 = entry_idx(e1);
-          select128<18, 1>(key, [&](int, int j) { return j < 16 ? xl + 64 * j : (j == 16 ? ri0 : ri1); },
-                           seed, bands, outs);
+          select128<18>(key, [&](int j) { return j < 16 ? xl + 64 * j : (j == 16 ? ri0 : ri1); },
+                        seed, cand, list[r]);
         }
       }
     }
@@ -204,32 +207,30 @@ __global__ __launch_bounds__(kThreads) void topk_merge_kernel(const entry_t* par
                                                               long long* indices, long long rows,
                                                               int parts, int k) {
   __shared__ entry_t list[4][kTop];
-  __shared__ entry_t bands[4][kTop];
+  __shared__ entry_t cands[4][kCand];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const long long row = (long long)blockIdx.x * 4 + wave;
   if (row >= rows) return;
   list[wave][lane] = 0ull;
   list[wave][lane + 64] = 0ull;
-  uint32_t seed[1] = {0u};
-  entry_t* const outs[1] = {list[wave]};
-  entry_t* const bnds[1] = {bands[wave]};
+  uint32_t seed = 0u;
   for (int p0 = 0; p0 < parts; p0 += 8) {
-    uint32_t key[1][18];
-    int idx[1][18];
+    uint32_t key[18];
+    int idx[18];
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       const int p = p0 + (j >> 1);
       const entry_t e = p < parts ? part[((long long)p * rows + row) * kTop + lane + 64 * (j & 1)] : 0ull;
-      key[0][j] = entry_key(e);
-      idx[0][j] = entry_idx(e);
+      key[j] = entry_key(e);
+      idx[j] = entry_idx(e);
     }
     const entry_t r0 = list[wave][lane], r1 = list[wave][lane + 64];
-    key[0][16] = entry_key(r0);
-    idx[0][16] = entry_idx(r0);
-    key[0][17] = entry_key(r1);
-    idx[0][17] = entry_idx(r1);
-    select128<18, 1>(key, [&](int, int j) { return idx[0][j]; }, seed, bnds, outs);
+    key[16] = entry_key(r0);
+    idx[16] = entry_idx(r0);
+    key[17] = entry_key(r1);
+    idx[17] = entry_idx(r1);
+    select128<18>(key, [&](int j) { return idx[j]; }, seed, cands[wave], list[wave]);
   }
   const entry_t* const lists[1] = {list[wave]};
   float* const cv[1] = {values + row * k};
@@ -242,34 +243,32 @@ __global__ __launch_bounds__(kThreads) void topk1d_partial_kernel(const float* a
                                                                   long long span, int parts,
                                                                   entry_t* part) {
   __shared__ entry_t list[4][kTop];
-  __shared__ entry_t bands[4][kTop];
+  __shared__ entry_t cands[4][kCand];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int p = blockIdx.x * 4 + wave;
   if (p >= parts) return;
   list[wave][lane] = 0ull;
   list[wave][lane + 64] = 0ull;
-  uint32_t seed[1] = {0u};
-  entry_t* const outs[1] = {list[wave]};
-  entry_t* const bnds[1] = {bands[wave]};
+  uint32_t seed = 0u;
   const long long begin = (long long)p * span;
   const long long end = begin + span < n ? begin + span : n;
   for (long long c0 = begin; c0 < end; c0 += 1024) {
-    uint32_t key[1][18];
-    int idx[1][18];
+    uint32_t key[18];
+    int idx[18];
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       const long long x = c0 + lane + 64 * j;
       const bool ok = x < end;
-      key[0][j] = ok ? f2key(arr[x]) : 0u;
-      idx[0][j] = (int)x;
+      key[j] = ok ? f2key(arr[x]) : 0u;
+      idx[j] = (int)x;
     }
     const entry_t r0 = list[wave][lane], r1 = list[wave][lane + 64];
-    key[0][16] = entry_key(r0);
-    idx[0][16] = entry_idx(r0);
-    key[0][17] = entry_key(r1);
-    idx[0][17] = entry_idx(r1);
-    select128<18, 1>(key, [&](int, int j) { return idx[0][j]; }, seed, bnds, outs);
+    key[16] = entry_key(r0);
+    idx[16] = entry_idx(r0);
+    key[17] = entry_key(r1);
+    idx[17] = entry_idx(r1);
+    select128<18>(key, [&](int j) { return idx[j]; }, seed, cands[wave], list[wave]);
   }
   const long long o = (long long)p * kTop;
   part[o + lane] = list[wave][lane];
