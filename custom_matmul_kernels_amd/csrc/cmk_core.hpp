@@ -1,7 +1,7 @@
 // Shared fp32-MFMA tiled GEMM core for gfx950 (CDNA4, wave64).
 //
-// One 256-thread work-group (4 waves) computes a TX x TY macro tile of the
-// product of two operands that both have a contraction axis k:
+// One work-group (4 or 8 waves) computes a TX x TY macro tile of the product
+// of two operands that both have a contraction axis k:
 //   X : TX "rows"  -> MFMA source A, the axis that ends up INSIDE a lane
 //   Y : TY "rows"  -> MFMA source B, the axis that ends up ACROSS lanes
 // Which matrix of the user's problem plays X and which plays Y is chosen by
@@ -9,19 +9,27 @@
 // axis in X (running state stays in one lane), a row-major store wants the
 // contiguous axis in Y (a store instruction writes 128-byte row segments).
 //
-// The contraction is walked in slabs of KS (32 unless a kernel asks otherwise).  A slab of each operand is
-// fetched from global memory into registers, written to one of two LDS
-// buffers, and consumed from the other with v_mfma_f32_32x32x2_f32.  Inside a
-// slab, k is consumed in groups of 8: lanes 0-31 feed k = 8g+0..3 and lanes
-// 32-63 feed k = 8g+4..7 of both operands, so one 128-bit LDS read per 32x32
-// block supplies four MFMA steps.  (A sum over k does not care about the
+// The contraction is walked in slabs of KS (32 unless a kernel asks
+// otherwise).  A slab of each operand travels from global memory straight into
+// one of two LDS buffers (global_load_lds_dwordx4: no registers, no LDS store
+// instructions) and is consumed from there with v_mfma_f32_32x32x2_f32.
+// Inside a slab, k is consumed in groups of 8: lanes 0-31 feed k = 8g+0..3 and
+// lanes 32-63 feed k = 8g+4..7 of both operands, so one 128-bit LDS read per
+// 32x32 block supplies four MFMA steps.  (A sum over k does not care about the
 // order, as long as both operands use the same one.)
 //
-// An operand tile can sit in memory, and in LDS, in one of two ways:
-//   KC : element(row, k) at row*ld + k   (k contiguous)  -> LDS [row][KS+4]
-//   RC : element(row, k) at k*ld + row   (rows contiguous) -> LDS [k][T+8]
-// Both are written with 128-bit stores straight from 128-bit global loads;
-// no transposition is needed on the way in.
+// An operand tile can sit in memory in one of two ways, and keeps that order
+// in LDS:
+//   KC : element(row, k) at row*ld + k   (k contiguous).  LDS holds rows of KS
+//        floats; the 16-byte chunk c of row r is stored at chunk c ^ (r & 7),
+//        so that the 128-bit fragment reads of 32 consecutive rows spread over
+//        all banks.
+//   RC : element(row, k) at k*ld + row   (rows contiguous).  LDS holds KS rows
+//        of T floats; fragment reads are four 32-bit reads down a column.
+// A direct load deposits lane i's 16 bytes at (instruction base + 16*i), so
+// the layout above is produced by choosing which global chunk each lane asks
+// for.  Tiles that touch the edge of a matrix (or are not 16-byte aligned) go
+// through registers instead: clamped scalar loads, zero fill, LDS stores.
 //
 // Plays the role of load_ab_*, buffer2smem_* and thread_matmul_* of the
 // reference (kernels/bmm_helpers.cu:114-164, 240-622).
@@ -37,8 +45,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // Operands live in global memory; loading through pointers that say so gives
 // global_load instructions (a generic pointer would give flat loads, which
 // also count against the LDS wait counter).
-typedef const f32x4 __attribute__((address_space(1))) * global_f32x4_ptr;
 typedef const float __attribute__((address_space(1))) * global_f32_ptr;
+typedef const void __attribute__((address_space(1))) * global_void_ptr;
+typedef void __attribute__((address_space(3))) * lds_void_ptr;
 
 constexpr int kThreads = 256;
 constexpr int KC = 0;   // k-contiguous operand
@@ -61,128 +70,51 @@ __device__ __forceinline__ P* uniform_ptr(P* p) {
   return reinterpret_cast<P*>((static_cast<unsigned long long>(hi) << 32) | lo);
 }
 
-// LDS footprint of one slab (KS deep) of a T-row operand tile.
+// Position (in floats) of element (row, k) of a T x KS operand tile in LDS.
 template <int KIND, int T, int KS>
-struct TileLayout;
-template <int T, int KS>
-struct TileLayout<KC, T, KS> {
-  static constexpr int pitch = KS + 4;
-  static constexpr int floats = T * pitch;
-};
-template <int T, int KS>
-struct TileLayout<RC, T, KS> {
-  static constexpr int pitch = T + 8;
-  static constexpr int floats = KS * pitch;
-};
+__device__ __forceinline__ int lds_pos(int row, int k) {
+  if constexpr (KIND == KC)
+    return row * KS + ((((k >> 2) ^ row) & 7) | ((k >> 2) & ~7)) * 4 + (k & 3);
+  else
+    return k * T + row;
+}
 
-// ---- global -> registers ---------------------------------------------------
-// Each of the NT threads fetches NV = T*KS/(4*NT) groups of four consecutive floats.  For
-// both kinds the element a thread fetches in pass p sits at
-//     tile + (t / TPR + p * RPP) * ld + (t % TPR) * 4
-// (KC: row-major rows x k, RC: k-major k x rows), so the per-lane part
-// `lane_off` is fixed for a whole kernel and everything else is scalar.
+// How the 1 KB pieces that one direct-load instruction moves are dealt to the
+// waves: piece q = p * NW + wave covers, for KC, 256/KS consecutive rows of
+// the tile and, for RC, 256 consecutive floats of the [KS][T] tile.
 template <int KIND, int T, int KS, int NT>
 struct LoadMap {
-  static constexpr int NV = T * KS / (NT * 4);             // float4 per thread
-  static constexpr int TPR = KIND == KC ? KS / 4 : T / 4;  // threads per contiguous run
-  static constexpr int RPP = NT / TPR;                     // runs per pass
-  static_assert(NV >= 1 && NV * NT * 4 == T * KS, "tile does not divide among the threads");
+  static constexpr int NW = NT / 64;
+  static constexpr int NI = T * KS / 256;     // pieces per tile
+  static constexpr int NV = NI / NW;          // pieces (instructions) per wave
+  static_assert(NV >= 1 && NV * NW == NI, "tile does not divide among the waves");
+  static_assert(KIND == RC || KS >= 32, "the chunk swizzle needs at least 8 chunks per row");
+  static_assert(KIND == KC || 256 % T == 0 || T % 256 == 0, "row-contiguous tile width");
 };
 
+// Byte offset, relative to the tile's first element in global memory, of the 16
+// bytes this lane fetches with its p-th direct load.
 template <int KIND, int T, int KS, int NT>
 __device__ __forceinline__ void lane_offsets_bytes(const Operand& o,
-                                                   unsigned (&off)[T * KS / (NT * 4)]) {
+                                                   unsigned (&off)[LoadMap<KIND, T, KS, NT>::NV]) {
   using M = LoadMap<KIND, T, KS, NT>;
-  const int t = threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
 #pragma unroll
-  for (int p = 0; p < M::NV; ++p)
-    off[p] = static_cast<unsigned>(((long long)(t / M::TPR + p * M::RPP) * o.ld + (t % M::TPR) * 4) * 4);
-}
-
-// r0, k0, K are wave-uniform.  A tile that lies completely inside the matrix
-// takes the branch-free path.
-template <int KIND, int T, int KS, int NT>
-__device__ __forceinline__ void gload(const Operand& o,
-                                      const unsigned (&lane_off)[T * KS / (NT * 4)], int r0, int k0,
-                                      int K, f32x4 (&v)[T * KS / (NT * 4)]) {
-  using M = LoadMap<KIND, T, KS, NT>;
-  constexpr int NV = M::NV, TPR = M::TPR, RPP = M::RPP;
-  const int t = threadIdx.x;
-  const bool interior = o.vec && (k0 + KS <= K) && (r0 + T <= o.rows) &&
-                        ((long long)(T + KS) * o.ld < (1ll << 29));
-  if (interior) {
-    const long long first = KIND == KC ? (long long)r0 * o.ld + k0 : (long long)k0 * o.ld + r0;
-    const char* tile = reinterpret_cast<const char*>(o.p + first);
-#pragma unroll
-    for (int p = 0; p < NV; ++p) v[p] = *(global_f32x4_ptr)(tile + lane_off[p]);
-  } else if (K > 0 && o.rows > 0) {
-    // edge tile: every element is fetched from a clamped (always valid)
-    // address and zeroed when it lies outside the matrix; no divergent branches
+  for (int p = 0; p < M::NV; ++p) {
+    const int q = p * M::NW + wave;
+    long long e;
     if constexpr (KIND == KC) {
-      const int kk = k0 + (t % TPR) * 4;
-      const int rr = r0 + t / TPR;
-#pragma unroll
-      for (int p = 0; p < NV; ++p) {
-        const int row = rr + RPP * p;
-        const float* src = o.p + (long long)row * o.ld + kk;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[p][j] = *(global_f32_ptr)((row < o.rows && kk + j < K) ? src + j : o.p);
-      }
-#pragma unroll
-      for (int p = 0; p < NV; ++p) {
-        const int row = rr + RPP * p;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[p][j] = (row < o.rows && kk + j < K) ? v[p][j] : 0.f;
-      }
+      constexpr int CPR = KS / 4;  // chunks per row
+      const int row = q * (256 / KS) + lane / CPR;
+      const int slot = lane % CPR;
+      const int chunk = ((slot ^ row) & 7) | (slot & ~7);
+      e = (long long)row * o.ld + chunk * 4;
     } else {
-      const int rr = r0 + (t % TPR) * 4;
-      const int kb = k0 + t / TPR;
-#pragma unroll
-      for (int p = 0; p < NV; ++p) {
-        const int kk = kb + p * RPP;
-        const float* src = o.p + (long long)kk * o.ld + rr;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[p][j] = *(global_f32_ptr)((kk < K && rr + j < o.rows) ? src + j : o.p);
-      }
-#pragma unroll
-      for (int p = 0; p < NV; ++p) {
-        const int kk = kb + p * RPP;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) v[p][j] = (kk < K && rr + j < o.rows) ? v[p][j] : 0.f;
-      }
+      const int f = q * 256 + lane * 4;  // float position inside the [KS][T] tile
+      e = (long long)(f / T) * o.ld + f % T;
     }
-  } else {
-#pragma unroll
-    for (int p = 0; p < NV; ++p) v[p] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-}
-
-// ---- registers -> LDS --------------------------------------------------------
-template <int KIND, int T, int KS, int NT>
-__device__ __forceinline__ void lstore(float* lds, const f32x4 (&v)[T * KS / (NT * 4)]) {
-  using M = LoadMap<KIND, T, KS, NT>;
-  const int t = threadIdx.x;
-  constexpr int pitch = TileLayout<KIND, T, KS>::pitch;
-#pragma unroll
-  for (int p = 0; p < M::NV; ++p)
-    *reinterpret_cast<f32x4*>(&lds[(t / M::TPR + p * M::RPP) * pitch + (t % M::TPR) * 4]) = v[p];
-}
-
-// ---- LDS -> MFMA fragment ----------------------------------------------------
-// Four k values (8*kg + 4*half + 0..3) of tile row `row` for this lane.
-template <int KIND, int T, int KS>
-__device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg, int half) {
-  constexpr int pitch = TileLayout<KIND, T, KS>::pitch;
-  if constexpr (KIND == KC) {
-    return *reinterpret_cast<const f32x4*>(&lds[row * pitch + kg * 8 + half * 4]);
-  } else {
-    const float* q = &lds[(kg * 8 + half * 4) * pitch + row];
-    f32x4 r;
-    r.x = q[0];
-    r.y = q[pitch];
-    r.z = q[2 * pitch];
-    r.w = q[3 * pitch];
-    return r;
+    off[p] = static_cast<unsigned>(e * 4);
   }
 }
 
@@ -191,12 +123,12 @@ __device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg, int hal
 //
 // The engine walks a flat sequence of slabs: `ntiles` consecutive X tiles
 // (starting at element `xbase`) against one Y strip, S = ceil(K/KS) slabs per
-// tile.  While slab i is multiplied, slab i+1 is written to the other LDS
-// buffer (in the middle of the slab) and slab i+2 is on its way from global
-// memory.  The one barrier per slab sits inside the last k-group; right after
-// it the first fragments of slab i+1 are read, so the matrix pipe keeps running
-// across slab and tile boundaries.  Inside a k-group all LDS and global traffic
-// is issued directly behind the group's first MFMA step, where it costs no
+// tile.  While slab i is multiplied, slab i+1 is landing in the other LDS
+// buffer.  The one barrier per slab sits inside the last k-group; right after
+// it the loads of slab i+2 are issued into the buffer that just became free
+// and the first fragments of slab i+1 are read, so the matrix pipe keeps
+// running across slab and tile boundaries.  Inside a k-group all LDS traffic is
+// issued directly behind the group's first MFMA step, where it costs no
 // matrix-pipe time.
 template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32>
 struct Core {
@@ -204,45 +136,124 @@ struct Core {
   static constexpr int NT = WX * WY * 64;      // threads per work-group
   static constexpr int KS = KS_;
   static constexpr int NG = KS / 8;            // k-groups per slab
-  static constexpr int WRITE_AT = NG / 2 - 1;  // k-group after which the next slab goes to LDS
   static constexpr int TX = WX * BX * 32;
   static constexpr int TY = WY * BY * 32;
   static_assert(NG >= 2 && NG % 2 == 0, "slab depth");
-  static constexpr int xFloats = TileLayout<XK, TX, KS>::floats;
-  static constexpr int yFloats = TileLayout<YK, TY, KS>::floats;
+  static constexpr int xFloats = TX * KS;
+  static constexpr int yFloats = TY * KS;
   static constexpr int bufFloats = xFloats + yFloats;
   static constexpr int ldsFloats = 2 * bufFloats;
+  using MX = LoadMap<XK, TX, KS, NT>;
+  using MY = LoadMap<YK, TY, KS, NT>;
 
-  f32x4 xv[TX * KS / (NT * 4)];  // slab in flight from global memory
-  f32x4 yv[TY * KS / (NT * 4)];
   f32x4 xf[2][BX];           // fragments; [0] holds k-group 0 of the current slab at slab entry
   f32x4 yf[2][BY];
   int it, iters, S;          // flat slab counter (wave-uniform)
   int lt, ls;                // (tile, slab) of the next slab to fetch (wave-uniform)
   int xbase, y0, K;
   int xr, yr, half;
-  unsigned xoff[TX * KS / (NT * 4)];  // this lane's byte offsets inside an operand tile
-  unsigned yoff[TY * KS / (NT * 4)];
+  unsigned xoff[MX::NV];     // this lane's byte offsets for the direct loads
+  unsigned yoff[MY::NV];
+  float* pend_buf;           // buffer whose Y half is still to be requested (wave-uniform)
+  int pend_k0;
 
-  __device__ __forceinline__ void load(const Operand& X, const Operand& Y) {
+  // One operand's slab -> LDS.  Interior tiles: NV direct loads per wave.  Edge
+  // tiles: every element is fetched from a clamped (always valid) address,
+  // zeroed when it lies outside the matrix, and stored from registers.
+  template <int KIND, int T, class M>
+  __device__ __forceinline__ void fetch(const Operand& o, const unsigned (&off)[M::NV], int r0,
+                                        int k0, float* dst) {
+    const bool interior = o.vec && (k0 + KS <= K) && (r0 + T <= o.rows) &&
+                          ((long long)(T + KS) * o.ld < (1ll << 29));
+    if (interior) {
+      const long long first = KIND == KC ? (long long)r0 * o.ld + k0 : (long long)k0 * o.ld + r0;
+      const char* tile = reinterpret_cast<const char*>(o.p + first);
+      const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+      for (int p = 0; p < M::NV; ++p)
+        __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + off[p]),
+                                         (lds_void_ptr)(dst + (p * M::NW + wave) * 256), 16, 0, 0);
+    } else {
+      // NT threads x 4 floats per pass, walking the tile in its memory order
+      constexpr int RUN = KIND == KC ? KS : T;        // contiguous floats per line
+      constexpr int TPR = RUN / 4;                    // threads per line
+      constexpr int LPP = NT / TPR;                   // lines per pass
+      constexpr int PASSES = (KIND == KC ? T : KS) / LPP;
+      static_assert(PASSES >= 1, "edge path shape");
+      const int t = threadIdx.x;
+      const int c4 = (t % TPR) * 4;
+      f32x4 v[PASSES];
+      const bool any = K > 0 && o.rows > 0;
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        const int line = t / TPR + p * LPP;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int rj = KIND == KC ? r0 + line : r0 + c4 + j;
+          const int kj = KIND == KC ? k0 + c4 + j : k0 + line;
+          const bool ok = any && rj < o.rows && kj < K;
+          const long long e = KIND == KC ? (long long)rj * o.ld + kj : (long long)kj * o.ld + rj;
+          v[p][j] = any ? *(global_f32_ptr)(ok ? o.p + e : o.p) : 0.f;
+        }
+      }
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        const int line = t / TPR + p * LPP;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int rj = KIND == KC ? r0 + line : r0 + c4 + j;
+          const int kj = KIND == KC ? k0 + c4 + j : k0 + line;
+          v[p][j] = (rj < o.rows && kj < K) ? v[p][j] : 0.f;
+        }
+        const int pos = KIND == KC ? lds_pos<KC, T, KS>(line, c4) : lds_pos<RC, T, KS>(c4, line);
+        *reinterpret_cast<f32x4*>(dst + pos) = v[p];
+      }
+    }
+  }
+
+  // Starts the transfer of the next slab of the sequence into `buf`: the X
+  // operand now, the Y operand one k-group later (issue_y), so that the waves'
+  // loads do not all queue up at the memory pipeline in the same few cycles.
+  __device__ __forceinline__ void issue_x(const Operand& X, float* buf) {
     // the slab coordinates are the same for every lane; saying so keeps the
     // address arithmetic on the scalar unit
     const int x0 = __builtin_amdgcn_readfirstlane(xbase + lt * TX);
-    const int k0 = __builtin_amdgcn_readfirstlane(ls * KS);
-    gload<XK, TX, KS, NT>(X, xoff, x0, k0, K, xv);
-    gload<YK, TY, KS, NT>(Y, yoff, y0, k0, K, yv);
+    pend_k0 = __builtin_amdgcn_readfirstlane(ls * KS);
+    pend_buf = buf;
+    fetch<XK, TX, MX>(X, xoff, x0, pend_k0, buf);
     if (++ls == S) { ls = 0; ++lt; }
   }
-  __device__ __forceinline__ void store(float* buf) {
-    lstore<XK, TX, KS, NT>(buf, xv);
-    lstore<YK, TY, KS, NT>(buf + xFloats, yv);
+  __device__ __forceinline__ void issue_y(const Operand& Y) {
+    if (pend_buf) fetch<YK, TY, MY>(Y, yoff, y0, pend_k0, pend_buf + xFloats);
+    pend_buf = nullptr;
   }
+
+  template <int KIND, int T>
+  __device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg) {
+    if constexpr (KIND == KC) {
+      return *reinterpret_cast<const f32x4*>(&lds[lds_pos<KC, T, KS>(row, kg * 8 + half * 4)]);
+    } else {
+      const float* q = &lds[(kg * 8 + half * 4) * T + row];
+      f32x4 r;
+      r.x = q[0];
+      r.y = q[T];
+      r.z = q[2 * T];
+      r.w = q[3 * T];
+      return r;
+    }
+  }
+  // Four k values (8*kg + 4*half + 0..3) of every block row of this lane.
   __device__ __forceinline__ void read_frags(const float* buf, int kg, f32x4 (&fx)[BX],
                                              f32x4 (&fy)[BY]) {
 #pragma unroll
-    for (int b = 0; b < BX; ++b) fx[b] = frag<XK, TX, KS>(buf, xr + 32 * b, kg, half);
+    for (int b = 0; b < BX; ++b) fx[b] = frag<XK, TX>(buf, xr + 32 * b, kg);
 #pragma unroll
-    for (int b = 0; b < BY; ++b) fy[b] = frag<YK, TY, KS>(buf + xFloats, yr + 32 * b, kg, half);
+    for (int b = 0; b < BY; ++b) fy[b] = frag<YK, TY>(buf + xFloats, yr + 32 * b, kg);
+  }
+
+  // Waits until this wave's direct loads have landed in LDS.
+  __device__ __forceinline__ void wait_loads() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), leave expcnt / lgkmcnt alone
   }
 
   // Fills the pipeline: slab 0 in LDS with its first fragments in registers,
@@ -264,19 +275,20 @@ struct Core {
     it = 0;
     lt = 0;
     ls = 0;
-    load(X, Y);
-    store(lds);
+    issue_x(X, lds);
+    issue_y(Y);
+    wait_loads();
     __syncthreads();
+    if (iters > 1) issue_x(X, lds + bufFloats);
     read_frags(lds, 0, xf[0], yf[0]);
-    if (iters > 1) load(X, Y);
   }
 
   // acc += the current tile's product: S slabs of the flat sequence.
   __device__ __forceinline__ void tile(const Operand& X, const Operand& Y, float* lds,
                                        f32x16 (&acc)[BX][BY]) {
     for (int s = 0; s < S; ++s) {
-      const float* cur = lds + (it & 1) * bufFloats;
-      float* nxt = lds + ((it + 1) & 1) * bufFloats;
+      float* cur = lds + (it & 1) * bufFloats;
+      const float* nxt = lds + ((it + 1) & 1) * bufFloats;
       const bool has1 = it + 1 < iters;
       const bool has2 = it + 2 < iters;
 #pragma unroll
@@ -290,15 +302,14 @@ struct Core {
             acc[bx][by] = __builtin_amdgcn_mfma_f32_32x32x2f32(
                 xf[kg & 1][bx][0], yf[kg & 1][by][0], acc[bx][by], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
+        if (kg == 0) issue_y(Y);
         if (kg + 1 < NG) {
           read_frags(cur, kg + 1, xf[(kg + 1) & 1], yf[(kg + 1) & 1]);
         } else if (has1) {
-          __syncthreads();
+          wait_loads();     // this wave's part of slab it+1 is in LDS
+          __syncthreads();  // everyone's is, and nobody reads `cur` any more
+          if (has2) issue_x(X, cur);
           read_frags(nxt, 0, xf[0], yf[0]);
-        }
-        if (kg == WRITE_AT) {
-          if (has1) store(nxt);
-          if (has2) load(X, Y);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
