@@ -1,6 +1,6 @@
 // Shared fp32-MFMA tiled GEMM core for gfx950 (CDNA4, wave64).
 //
-// One work-group (4 or 8 waves) computes a TX x TY macro tile of the product
+// One work-group (4, 8 or 16 waves) computes a TX x TY macro tile of the product
 // of two operands that both have a contraction axis k:
 //   X : TX "rows"  -> MFMA source A, the axis that ends up INSIDE a lane
 //   Y : TY "rows"  -> MFMA source B, the axis that ends up ACROSS lanes
@@ -86,8 +86,9 @@ template <int KIND, int T, int KS, int NT>
 struct LoadMap {
   static constexpr int NW = NT / 64;
   static constexpr int NI = T * KS / 256;     // pieces per tile
-  static constexpr int NV = NI / NW;          // pieces (instructions) per wave
-  static_assert(NV >= 1 && NV * NW == NI, "tile does not divide among the waves");
+  static constexpr int NV = (NI + NW - 1) / NW;  // pieces (instructions) per wave
+  static constexpr bool kEven = NV * NW == NI;   // otherwise only pieces q < NI exist
+  static_assert(NI >= 1, "tile smaller than one piece");
   static_assert(KIND == RC || KS >= 32, "the chunk swizzle needs at least 8 chunks per row");
   static_assert(KIND == KC || 256 % T == 0 || T % 256 == 0, "row-contiguous tile width");
 };
@@ -118,7 +119,7 @@ __device__ __forceinline__ void lane_offsets_bytes(const Operand& o,
   }
 }
 
-// Work-group level tile engine.  WX x WY waves (4 or 8 of them), each wave owns
+// Work-group level tile engine.  WX x WY waves (4, 8 or 16 of them), each wave owns
 // BX x BY blocks of 32x32; KS is the contraction depth of one LDS slab.
 //
 // The engine walks a flat sequence of slabs: `ntiles` consecutive X tiles
@@ -132,7 +133,7 @@ __device__ __forceinline__ void lane_offsets_bytes(const Operand& o,
 // matrix-pipe time.
 template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32>
 struct Core {
-  static_assert(WX * WY == 4 || WX * WY == 8, "four or eight waves per work-group");
+  static_assert(WX * WY == 4 || WX * WY == 8 || WX * WY == 16, "4, 8 or 16 waves per work-group");
   static constexpr int NT = WX * WY * 64;      // threads per work-group
   static constexpr int KS = KS_;
   static constexpr int NG = KS / 8;            // k-groups per slab
@@ -171,15 +172,17 @@ struct Core {
       const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 #pragma unroll
       for (int p = 0; p < M::NV; ++p)
-        __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + off[p]),
-                                         (lds_void_ptr)(dst + (p * M::NW + wave) * 256), 16, 0, 0);
+        if (M::kEven || p * M::NW + wave < M::NI)
+          __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + off[p]),
+                                           (lds_void_ptr)(dst + (p * M::NW + wave) * 256), 16, 0, 0);
     } else {
       // NT threads x 4 floats per pass, walking the tile in its memory order
       constexpr int RUN = KIND == KC ? KS : T;        // contiguous floats per line
       constexpr int TPR = RUN / 4;                    // threads per line
       constexpr int LPP = NT / TPR;                   // lines per pass
-      constexpr int PASSES = (KIND == KC ? T : KS) / LPP;
-      static_assert(PASSES >= 1, "edge path shape");
+      constexpr int LINES = KIND == KC ? T : KS;
+      constexpr int PASSES = (LINES + LPP - 1) / LPP;
+      constexpr bool kAllLines = PASSES * LPP == LINES;  // otherwise some threads have no line
       const int t = threadIdx.x;
       const int c4 = (t % TPR) * 4;
       f32x4 v[PASSES];
@@ -191,7 +194,7 @@ struct Core {
         for (int j = 0; j < 4; ++j) {
           const int rj = KIND == KC ? r0 + line : r0 + c4 + j;
           const int kj = KIND == KC ? k0 + c4 + j : k0 + line;
-          const bool ok = any && rj < o.rows && kj < K;
+          const bool ok = any && rj < o.rows && kj < K && (kAllLines || line < LINES);
           const long long e = KIND == KC ? (long long)rj * o.ld + kj : (long long)kj * o.ld + rj;
           v[p][j] = any ? *(global_f32_ptr)(ok ? o.p + e : o.p) : 0.f;
         }
@@ -206,7 +209,7 @@ struct Core {
           v[p][j] = (rj < o.rows && kj < K) ? v[p][j] : 0.f;
         }
         const int pos = KIND == KC ? lds_pos<KC, T, KS>(line, c4) : lds_pos<RC, T, KS>(c4, line);
-        *reinterpret_cast<f32x4*>(dst + pos) = v[p];
+        if (kAllLines || line < LINES) *reinterpret_cast<f32x4*>(dst + pos) = v[p];
       }
     }
   }

@@ -1,16 +1,18 @@
 // Wave-level exact top-128 selection and a wave64 bitonic sorter.
 //
-// A wave holds NR*64 candidates of one output row, NR per lane, as 32-bit
-// order-preserving keys plus 32-bit indices.  select128() finds the 128 largest
-// in three moves:
+// A wave holds NR*64 candidates of one output row, NR per lane, as fp32 bit
+// patterns; their order is that of 32-bit order-preserving keys.  select128()
+// finds the 128 largest in three moves:
 //   1. Bracket the key of the 128th largest, [lo, hi), by counting candidates
-//      >= t with wave ballots.  The bracket starts around the previous row's
-//      answer (rows of one strip are statistically alike) and is bisected until
-//      at most 256 candidates lie at or above lo.
-//   2. One pass over the registers compacts those candidates into a list in
-//      LDS, as 64-bit (key, ~index) entries.
-//   3. The list, now four entries per lane, is bisected to the exact threshold
-//      and the 128 winners are written to the output list.
+//      >= t with wave ballots.  The bracket starts just below the previous
+//      row's answer (rows of one strip are statistically alike), which is
+//      nearly always right at once; otherwise it is bisected until at most 256
+//      candidates lie at or above lo.
+//   2. The ballots of the last count compact those candidates into a list in
+//      LDS, as 64-bit (raw, ~index) entries.
+//   3. The list, now four entries per lane and turned into keys, is narrowed
+//      four-fold per round to the exact threshold and the 128 winners are
+//      written to the output list as (key, ~index) entries.
 // The output list is unordered; bitonic128_desc() orders it once, at the very
 // end, so that values descend and equal values come out by ascending index.
 //
@@ -26,10 +28,10 @@ namespace cmk {
 
 // Monotone map float -> uint32: a < b  <=>  key(a) < key(b) (with -0 < +0 and
 // NaNs at the extremes).  Key 0 is reserved for "no candidate".
-__device__ __forceinline__ uint32_t f2key(float f) {
-  const uint32_t u = __float_as_uint(f);
+__device__ __forceinline__ uint32_t raw2key(uint32_t u) {
   return u ^ (static_cast<uint32_t>(static_cast<int32_t>(u) >> 31) | 0x80000000u);
 }
+__device__ __forceinline__ uint32_t f2key(float f) { return raw2key(__float_as_uint(f)); }
 __device__ __forceinline__ float key2f(uint32_t k) {
   if (k == 0) return -__builtin_inff();
   const uint32_t u = (k & 0x80000000u) ? (k ^ 0x80000000u) : ~k;
@@ -61,95 +63,142 @@ __device__ __forceinline__ uint32_t bracket_mid(uint32_t lo, uint32_t hi) {
 
 constexpr int kCand = 256;  // capacity of the candidate list select128() works in
 
-// Selects the 128 largest keys among key[0..NR) of all 64 lanes and writes them
-// as entries to out[0..128) (LDS owned by this wave).  `cand` is kCand entries of
-// wave-private LDS scratch.  `seed` carries the threshold key from one call to
-// the next (0 = none); idx_of(j) is the index of candidate key[j] of this lane.
-// Ties at the threshold: earliest (register, lane) position first.  Fewer than
-// 128 real candidates leave empty entries.
+// Candidates travel as raw fp32 bit patterns ("raw") until they reach the
+// candidate list; comparing raws against a threshold key needs no key per
+// candidate:  key(raw) >= t  <=>  (int)raw >= (int)(t ^ 0x80000000)  for t in the
+// upper half of the key space, and  raw <= ~t  (unsigned) below it.  raw
+// 0xFFFFFFFF has key 0 and stands for "no candidate".
+constexpr uint32_t kNoCandidate = 0xFFFFFFFFu;
+__device__ __forceinline__ uint32_t key2raw(uint32_t k) {
+  return (k & 0x80000000u) ? (k ^ 0x80000000u) : ~k;
+}
+
+// m[j] = lanes whose raw[j] has a key >= t; returns how many there are.
+template <int NR>
+__device__ __forceinline__ int masks_ge(const uint32_t (&raw)[NR], uint32_t t,
+                                        unsigned long long (&m)[NR]) {
+  int c = 0;
+  if (t & 0x80000000u) {
+    const int b = static_cast<int>(t ^ 0x80000000u);
+#pragma unroll
+    for (int j = 0; j < NR; ++j) m[j] = __ballot(static_cast<int>(raw[j]) >= b);
+  } else {
+    const uint32_t b = ~t;
+#pragma unroll
+    for (int j = 0; j < NR; ++j) m[j] = __ballot(raw[j] <= b);
+  }
+#pragma unroll
+  for (int j = 0; j < NR; ++j) c += __popcll(m[j]);
+  return c;
+}
+
+// Selects the 128 candidates with the largest keys among raw[0..NR) of all 64
+// lanes and writes them as entries to out[0..128) (LDS owned by this wave).
+// `cand` is kCand entries of wave-private LDS scratch.  `seed` carries the
+// threshold key from one call to the next (0 = none); idx_of(j) is the index of
+// candidate raw[j] of this lane.  Ties at the threshold: earliest (register,
+// lane) position first.  Fewer than 128 real candidates leave empty entries.
 template <int NR, class IdxOf>
-__device__ __forceinline__ void select128(const uint32_t (&key)[NR], IdxOf&& idx_of,
+__device__ __forceinline__ void select128(const uint32_t (&raw)[NR], IdxOf&& idx_of,
                                           uint32_t& seed, entry_t* cand, entry_t* out) {
   const int lane = threadIdx.x & 63;
-  auto count_ge = [&](uint32_t t) {
-    int c = 0;
-#pragma unroll
-    for (int j = 0; j < NR; ++j) c += __popcll(__ballot(key[j] >= t));
-    return c;
-  };
-  // bracket: count(>= lo) >= 128 > count(>= hi); hi == 0 stands for 2^32
-  uint32_t lo = 0, hi = 0;
-  int c_lo = NR * 64, c_hi = 0;
+  constexpr uint32_t D = 1u << 20;  // +-12% of a float's magnitude
+  // bracket: count(>= lo) >= 128 > count(>= hi); hi == 0 stands for 2^32.
+  // m[] always holds the masks of the last threshold counted.
+  unsigned long long m[NR];
+  uint32_t lo = 0, hi = 0, counted = 0xFFFFFFFFu;
+  int c_lo = NR * 64;
   if (seed) {
-    constexpr uint32_t D = 1u << 20;  // +-12% of a float's magnitude
     const uint32_t t0 = seed > D ? seed - D : 1u;
-    const int c0 = count_ge(t0);
-    if (c0 >= kTop) { lo = t0; c_lo = c0; } else { hi = t0; c_hi = c0; }
-    if (hi == 0 && seed < 0xFFFFFFFFu - D) {
-      const uint32_t t1 = seed + D;
-      const int c1 = count_ge(t1);
-      if (c1 >= kTop) { lo = t1; c_lo = c1; } else { hi = t1; c_hi = c1; }
-    }
+    const int c0 = masks_ge(raw, t0, m);
+    counted = t0;
+    if (c0 >= kTop) { lo = t0; c_lo = c0; } else { hi = t0; }
   }
   while (c_lo > kCand && hi - lo != 1u) {
     const uint32_t mid = bracket_mid(lo, hi);
-    const int c = count_ge(mid);
-    if (c >= kTop) { lo = mid; c_lo = c; } else { hi = mid; c_hi = c; }
+    const int c = masks_ge(raw, mid, m);
+    counted = mid;
+    if (c >= kTop) { lo = mid; c_lo = c; } else { hi = mid; }
   }
 
   if (c_lo <= kCand) {
-    // one pass: every candidate >= lo goes to the candidate list, in (register,
-    // lane) order; there are at least 128 and at most 256 of them
-    int base = 0;
+    if (counted != lo) masks_ge(raw, lo, m);
+    // every candidate with a key >= lo goes to the candidate list, in (register,
+    // lane) order, as (raw, ~index); there are at least 128 and at most 256
+    int base[NR];
+    base[0] = 0;
+#pragma unroll
+    for (int j = 1; j < NR; ++j) base[j] = base[j - 1] + __popcll(m[j - 1]);
 #pragma unroll
     for (int j = 0; j < NR; ++j) {
-      const bool ge = key[j] >= lo;
-      const unsigned long long m = __ballot(ge);
-      const int pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m >> 32),
-                                                __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m), base));
-      if (ge) cand[pos] = pack_entry(key[j], idx_of(j));
-      base += __popcll(m);
+      const int pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m[j] >> 32),
+                                                __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m[j]), base[j]));
+      if (__builtin_amdgcn_inverse_ballot_w64(m[j])) cand[pos] = pack_entry(raw[j], idx_of(j));
     }
-    // four entries per lane; bisect to the exact threshold: the largest t with
-    // count(>= t) >= 128, stopping early when the count is exactly 128
+    // four entries per lane, now with keys
     entry_t e[4];
     uint32_t k[4];
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const bool valid = lane + 64 * m < c_lo;
-      e[m] = valid ? cand[lane + 64 * m] : 0ull;
-      k[m] = entry_key(e[m]);
-      if (k[m] == 0u) e[m] = 0ull;  // "no candidate" carries index -1
+    for (int q = 0; q < 4; ++q) {
+      const bool valid = lane + 64 * q < c_lo;
+      const entry_t r = cand[lane + 64 * q];
+      k[q] = valid ? raw2key(entry_key(r)) : 0u;
+      e[q] = k[q] ? (static_cast<entry_t>(k[q]) << 32) | static_cast<uint32_t>(r) : 0ull;
     }
-    int n_lo = c_lo;
-    while (n_lo != kTop && hi - lo != 1u) {
-      const uint32_t mid = bracket_mid(lo, hi);
+    auto count4 = [&](uint32_t t) {
       int c = 0;
 #pragma unroll
-      for (int m = 0; m < 4; ++m) c += __popcll(__ballot(lane + 64 * m < c_lo && k[m] >= mid));
-      if (c >= kTop) { lo = mid; n_lo = c; } else { hi = mid; }
+      for (int q = 0; q < 4; ++q) c += __popcll(__ballot(k[q] >= t));
+      return c;
+    };
+    int n_lo = c_lo;
+    // the upper end of the bracket, if still open, comes from the seed as well
+    if (hi == 0 && seed && seed < 0xFFFFFFFFu - D && seed + D > lo) {
+      const uint32_t t1 = seed + D;
+      const int c1 = count4(t1);
+      if (c1 >= kTop) { lo = t1; n_lo = c1; } else { hi = t1; }
+    }
+    // narrow the bracket four-fold per round to the exact threshold: the largest
+    // t with count(>= t) >= 128; stop early when a count is exactly 128
+    while (n_lo != kTop && hi - lo != 1u) {
+      const uint32_t w = hi - lo;
+      uint32_t q = w ? w >> 2 : 0x40000000u;
+      if (q == 0) q = 1;
+      uint32_t t1 = lo + q, t2 = t1 + q, t3 = t2 + q;
+      if (t2 < t1) t2 = 0xFFFFFFFFu;
+      if (t3 < t2) t3 = 0xFFFFFFFFu;
+      int c1 = 0, c2 = 0, c3 = 0;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        c1 += __popcll(__ballot(k[r] >= t1));
+        c2 += __popcll(__ballot(k[r] >= t2));
+        c3 += __popcll(__ballot(k[r] >= t3));
+      }
+      if (c3 >= kTop) { lo = t3; n_lo = c3; }
+      else if (c2 >= kTop) { lo = t2; n_lo = c2; hi = t3; }
+      else if (c1 >= kTop) { lo = t1; n_lo = c1; hi = t2; }
+      else { hi = t1; }
     }
     // winners: all entries >= lo if that is exactly 128, otherwise (ties at lo)
     // those above lo and then the first ones equal to lo
     const bool exact = n_lo == kTop;
-    int pos_gt = 0;
     unsigned long long mg[4];
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const bool valid = lane + 64 * m < c_lo;
-      const bool g = valid && (exact ? k[m] >= lo : k[m] > lo);
-      mg[m] = __ballot(g);
-      if (g) out[pos_gt + prefix_in(mg[m])] = e[m];
-      pos_gt += __popcll(mg[m]);
+    for (int q = 0; q < 4; ++q) mg[q] = __ballot(exact ? k[q] >= lo : k[q] > lo);
+    int pos_gt = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (__builtin_amdgcn_inverse_ballot_w64(mg[q])) out[pos_gt + prefix_in(mg[q])] = e[q];
+      pos_gt += __popcll(mg[q]);
     }
     if (!exact) {
       int pos_eq = pos_gt;
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const bool q = lane + 64 * m < c_lo && k[m] == lo;
-        const unsigned long long mq = __ballot(q);
+      for (int q = 0; q < 4; ++q) {
+        const bool tie = k[q] == lo;
+        const unsigned long long mq = __ballot(tie);
         const int p = pos_eq + prefix_in(mq);
-        if (q && p < kTop) out[p] = e[m];
+        if (tie && p < kTop) out[p] = e[q];
         pos_eq += __popcll(mq);
       }
     }
@@ -159,18 +208,19 @@ __device__ __forceinline__ void select128(const uint32_t (&key)[NR], IdxOf&& idx
     int base = 0;
 #pragma unroll
     for (int j = 0; j < NR; ++j) {
-      const bool g = key[j] > lo;
-      const unsigned long long m = __ballot(g);
-      if (g) out[base + prefix_in(m)] = pack_entry(key[j], idx_of(j));
-      base += __popcll(m);
+      const uint32_t key = raw2key(raw[j]);
+      const bool g = key > lo;
+      const unsigned long long mm = __ballot(g);
+      if (g) out[base + prefix_in(mm)] = pack_entry(key, idx_of(j));
+      base += __popcll(mm);
     }
 #pragma unroll
     for (int j = 0; j < NR; ++j) {
-      const bool q = key[j] == lo;
-      const unsigned long long m = __ballot(q);
-      const int p = base + prefix_in(m);
-      if (q && p < kTop) out[p] = lo ? pack_entry(lo, idx_of(j)) : 0ull;
-      base += __popcll(m);
+      const bool tie = raw2key(raw[j]) == lo;
+      const unsigned long long mm = __ballot(tie);
+      const int p = base + prefix_in(mm);
+      if (tie && p < kTop) out[p] = lo ? pack_entry(lo, idx_of(j)) : 0ull;
+      base += __popcll(mm);
     }
   }
   seed = lo;
@@ -258,9 +308,8 @@ __device__ __forceinline__ void bitonic128_desc(entry_t (&e0)[R], entry_t (&e1)[
 // Sorts R 128-entry lists and writes the first k entries of each as fp32
 // values and int64 indices; a null values[r] skips the store of that row.
 template <int R>
-__device__ __forceinline__ void sort_and_store(const entry_t* const (&list)[R],
-                                               float* const (&values)[R],
-                                               long long* const (&indices)[R], int k) {
+__device__ __forceinline__ void sort_and_store(const entry_t* const* list, float* const* values,
+                                               long long* const* indices, int k) {
   const int lane = threadIdx.x & 63;
   entry_t e0[R], e1[R];
 #pragma unroll

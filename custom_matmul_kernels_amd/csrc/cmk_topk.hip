@@ -48,8 +48,8 @@ template <int XK, int YK, bool MULTI>
 __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   // eight waves: wave % 4 picks 32 of a tile's 128 candidates, wave / 4 one of
   // the two 32-row halves of the strip.  One work-group per CU; its two waves
-  // per SIMD are always in the same phase, because on this part a wave's
-  // selection (VALU) work does not hide behind another wave's MFMA stream.
+  // per SIMD are always in the same phase, because on this part vector
+  // instructions of one wave do not issue while another wave of the SIMD streams MFMAs.
   using C = Core<XK, YK, 4, 2, 1, 1, MULTI ? 32 : 64>;
   static_assert(C::TX == 128 && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
   constexpr int stageFloats = kPassRows * kStagePitch;
@@ -142,14 +142,14 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
         if (y0 + r >= Yext) continue;
         const float* src = lds + pr * kStagePitch;
         const int xl = xc0 + lane;
-        uint32_t key[18];
+        uint32_t key[18];  // fp32 bit patterns
         if (xc0 + 1024 <= x_limit) {
 #pragma unroll
-          for (int j = 0; j < 16; ++j) key[j] = f2key(src[lane + 64 * j]);
+          for (int j = 0; j < 16; ++j) key[j] = __float_as_uint(src[lane + 64 * j]);
         } else {
 #pragma unroll
           for (int j = 0; j < 16; ++j)
-            key[j] = xl + 64 * j < x_limit ? f2key(src[lane + 64 * j]) : 0u;
+            key[j] = xl + 64 * j < x_limit ? __float_as_uint(src[lane + 64 * j]) : kNoCandidate;
         }
         if (!MULTI || xt0 == xt_begin) {
           // first chunk: the running list is empty
@@ -159,8 +159,8 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
           select128<16>(k16, [&](int j) { return xl + 64 * j; }, seed, cand, list[r]);
         } else {
           const entry_t e0 = list[r][lane], e1 = list[r][lane + 64];
-          key[16] = entry_key(e0);
-          key[17] = entry_key(e1);
+          key[16] = key2raw(entry_key(e0));
+          key[17] = key2raw(entry_key(e1));
           const int ri0 = entry_idx(e0), ri1 = entry_idx(e1);
           select128<18>(key, [&](int j) { return j < 16 ? xl + 64 * j : (j == 16 ? ri0 : ri1); },
                         seed, cand, list[r]);
@@ -216,19 +216,19 @@ __global__ __launch_bounds__(kThreads) void topk_merge_kernel(const entry_t* par
   list[wave][lane + 64] = 0ull;
   uint32_t seed = 0u;
   for (int p0 = 0; p0 < parts; p0 += 8) {
-    uint32_t key[18];
+    uint32_t key[18];  // fp32 bit patterns
     int idx[18];
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       const int p = p0 + (j >> 1);
       const entry_t e = p < parts ? part[((long long)p * rows + row) * kTop + lane + 64 * (j & 1)] : 0ull;
-      key[j] = entry_key(e);
+      key[j] = key2raw(entry_key(e));
       idx[j] = entry_idx(e);
     }
     const entry_t r0 = list[wave][lane], r1 = list[wave][lane + 64];
-    key[16] = entry_key(r0);
+    key[16] = key2raw(entry_key(r0));
     idx[16] = entry_idx(r0);
-    key[17] = entry_key(r1);
+    key[17] = key2raw(entry_key(r1));
     idx[17] = entry_idx(r1);
     select128<18>(key, [&](int j) { return idx[j]; }, seed, cands[wave], list[wave]);
   }
@@ -254,19 +254,19 @@ __global__ __launch_bounds__(kThreads) void topk1d_partial_kernel(const float* a
   const long long begin = (long long)p * span;
   const long long end = begin + span < n ? begin + span : n;
   for (long long c0 = begin; c0 < end; c0 += 1024) {
-    uint32_t key[18];
+    uint32_t key[18];  // fp32 bit patterns
     int idx[18];
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       const long long x = c0 + lane + 64 * j;
       const bool ok = x < end;
-      key[j] = ok ? f2key(arr[x]) : 0u;
+      key[j] = ok ? __float_as_uint(arr[x]) : kNoCandidate;
       idx[j] = (int)x;
     }
     const entry_t r0 = list[wave][lane], r1 = list[wave][lane + 64];
-    key[16] = entry_key(r0);
+    key[16] = key2raw(entry_key(r0));
     idx[16] = entry_idx(r0);
-    key[17] = entry_key(r1);
+    key[17] = key2raw(entry_key(r1));
     idx[17] = entry_idx(r1);
     select128<18>(key, [&](int j) { return idx[j]; }, seed, cands[wave], list[wave]);
   }
