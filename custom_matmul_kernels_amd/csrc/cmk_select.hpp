@@ -78,6 +78,7 @@ template <int NR>
 __device__ __forceinline__ int masks_ge(const uint32_t (&raw)[NR], uint32_t t,
                                         unsigned long long (&m)[NR]) {
   int c = 0;
+  t = __builtin_amdgcn_readfirstlane(t);  // the same in every lane: the ballots stay scalar
   if (t & 0x80000000u) {
     const int b = static_cast<int>(t ^ 0x80000000u);
 #pragma unroll
@@ -102,17 +103,25 @@ template <int NR, class IdxOf>
 __device__ __forceinline__ void select128(const uint32_t (&raw)[NR], IdxOf&& idx_of,
                                           uint32_t& seed, entry_t* cand, entry_t* out) {
   const int lane = threadIdx.x & 63;
-  constexpr uint32_t D = 1u << 20;  // +-12% of a float's magnitude
+  constexpr uint32_t D = 1u << 21;  // a quarter of a binade: 12 to 25% of a float's magnitude
   // bracket: count(>= lo) >= 128 > count(>= hi); hi == 0 stands for 2^32.
   // m[] always holds the masks of the last threshold counted.
   unsigned long long m[NR];
   uint32_t lo = 0, hi = 0, counted = 0xFFFFFFFFu;
   int c_lo = NR * 64;
+  seed = __builtin_amdgcn_readfirstlane(seed);
   if (seed) {
-    const uint32_t t0 = seed > D ? seed - D : 1u;
-    const int c0 = masks_ge(raw, t0, m);
-    counted = t0;
-    if (c0 >= kTop) { lo = t0; c_lo = c0; } else { hi = t0; }
+    // walk down from the seed, in growing steps, until at least 128 candidates
+    // lie at or above; the first step nearly always does it
+    uint32_t t = seed, step = D;
+    while (t > step) {
+      t -= step;
+      const int c = masks_ge(raw, t, m);
+      counted = t;
+      if (c >= kTop) { lo = t; c_lo = c; break; }
+      hi = t;
+      if (step < (1u << 29)) step <<= 2;
+    }
   }
   while (c_lo > kCand && hi - lo != 1u) {
     const uint32_t mid = bracket_mid(lo, hi);
@@ -152,11 +161,18 @@ __device__ __forceinline__ void select128(const uint32_t (&raw)[NR], IdxOf&& idx
       return c;
     };
     int n_lo = c_lo;
-    // the upper end of the bracket, if still open, comes from the seed as well
-    if (hi == 0 && seed && seed < 0xFFFFFFFFu - D && seed + D > lo) {
-      const uint32_t t1 = seed + D;
-      const int c1 = count4(t1);
-      if (c1 >= kTop) { lo = t1; n_lo = c1; } else { hi = t1; }
+    // the upper end of the bracket, if still open, is found by walking up from
+    // the seed in the same way
+    if (hi == 0 && seed) {
+      uint32_t t = seed > lo ? seed : lo, step = D;
+      while (t < 0xFFFFFFFFu - step) {
+        t += step;
+        const int c = count4(t);
+        if (c < kTop) { hi = t; break; }
+        lo = t;
+        n_lo = c;
+        if (step < (1u << 29)) step <<= 2;
+      }
     }
     // narrow the bracket four-fold per round to the exact threshold: the largest
     // t with count(>= t) >= 128; stop early when a count is exactly 128
