@@ -22,8 +22,9 @@
 
 namespace cmk {
 
-constexpr int kChunkTiles = 8;                 // tiles of 128 candidates per chunk
-constexpr int kStagePitch = 128 * kChunkTiles + 8;
+constexpr int kTileX = 256;                    // candidates per tile
+constexpr int kChunkTiles = 4;                 // tiles per chunk: 1024 candidates
+constexpr int kStagePitch = kTileX * kChunkTiles + 8;
 
 struct TopkArgs {
   Operand X, Y;
@@ -50,8 +51,8 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   // the two 32-row halves of the strip.  One work-group per CU; its two waves
   // per SIMD are always in the same phase, because on this part vector
   // instructions of one wave do not issue while another wave of the SIMD streams MFMAs.
-  using C = Core<XK, YK, 4, 2, 1, 1, MULTI ? 32 : 64>;
-  static_assert(C::TX == 128 && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
+  using C = Core<XK, YK, 4, 2, 2, 1, 32>;
+  static_assert(C::TX == kTileX && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
   constexpr int stageFloats = kPassRows * kStagePitch;
   constexpr int bandFloats = 8 * kCand * 2;  // one candidate list per wave
   constexpr int listFloats = kStripRows * kTop * 2;
@@ -108,11 +109,11 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
     const int nt = min(kChunkTiles, xt_end - xt0);
     __syncthreads();  // previous chunk's staging reads are finished
     core.begin(X, Y, xt0 * C::TX, y0, a.K, nt, lds);
-    f32x16 acc[kChunkTiles][1][1];
+    f32x16 acc[kChunkTiles][2][1];
 #pragma unroll
     for (int i = 0; i < kChunkTiles; ++i) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][0][0][r] = 0.f;
+      for (int r = 0; r < 16; ++r) acc[i][0][0][r] = acc[i][1][0][r] = 0.f;
       if (i < nt) core.tile(X, Y, lds, acc[i]);
     }
     __syncthreads();  // all fragment reads are done; the buffers become the staging area
@@ -124,15 +125,17 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
       if (g) __syncthreads();  // previous pass has been read
       // rows 16g .. 16g+15 live in the waves with wy == g / 2, lanes l32 / 16 == g % 2
       if (wy == (g >> 1) && (l32 >> 4) == (g & 1)) {
-        float* row = lds + (l32 & 15) * kStagePitch + wx * 32 + 4 * half;
+        float* row = lds + (l32 & 15) * kStagePitch + wx * 64 + 4 * half;
 #pragma unroll
         for (int i = 0; i < kChunkTiles; ++i)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            f32x4 v = {acc[i][0][0][4 * q], acc[i][0][0][4 * q + 1], acc[i][0][0][4 * q + 2],
-                       acc[i][0][0][4 * q + 3]};
-            *reinterpret_cast<f32x4*>(row + i * 128 + 8 * q) = v;
-          }
+          for (int bx = 0; bx < 2; ++bx)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              f32x4 v = {acc[i][bx][0][4 * q], acc[i][bx][0][4 * q + 1], acc[i][bx][0][4 * q + 2],
+                         acc[i][bx][0][4 * q + 3]};
+              *reinterpret_cast<f32x4*>(row + i * kTileX + bx * 32 + 8 * q) = v;
+            }
       }
       __syncthreads();
 #pragma unroll 1
@@ -278,7 +281,7 @@ __global__ __launch_bounds__(kThreads) void topk1d_partial_kernel(const float* a
 static void plan_topk(int L, int Xext, int Yext, int* ystrips, int* xtiles, int* splits,
                       int* tiles_per_split) {
   *ystrips = ceil_div(Yext, kStripRows);
-  *xtiles = ceil_div(Xext, 128);
+  *xtiles = ceil_div(Xext, kTileX);
   const long long strips = (long long)L * *ystrips;
   const int chunks = ceil_div(*xtiles, kChunkTiles);
   int want = 1;
