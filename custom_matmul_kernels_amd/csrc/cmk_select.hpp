@@ -321,31 +321,159 @@ __device__ __forceinline__ void bitonic128_desc(entry_t (&e0)[R], entry_t (&e1)[
   bitonic_merge<128, 64, R>(e0, e1);
 }
 
-// Sorts R 128-entry lists and writes the first k entries of each as fp32
-// values and int64 indices; a null values[r] skips the store of that row.
-template <int R>
-__device__ __forceinline__ void sort_and_store(const entry_t* const* list, float* const* values,
-                                               long long* const* indices, int k) {
-  const int lane = threadIdx.x & 63;
-  entry_t e0[R], e1[R];
+// The same network on bare keys.
+template <int SIZE, int STRIDE, int R>
+__device__ __forceinline__ void key_stage(uint32_t (&k0)[R], uint32_t (&k1)[R]) {
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    e0[r] = list[r][lane];
-    e1[r] = list[r][lane + 64];
+    if constexpr (STRIDE == 64) {
+      const uint32_t hi = max(k0[r], k1[r]);
+      const uint32_t lo = min(k0[r], k1[r]);
+      k0[r] = hi;
+      k1[r] = lo;
+    } else {
+      const uint32_t o0 = lane_xor<STRIDE>(k0[r]);
+      const uint32_t o1 = lane_xor<STRIDE>(k1[r]);
+      constexpr unsigned long long km0 = keep_max_mask<SIZE, STRIDE, 0>();
+      constexpr unsigned long long km1 = keep_max_mask<SIZE, STRIDE, 1>();
+      const bool t0 = __builtin_amdgcn_inverse_ballot_w64(__ballot(o0 > k0[r]) ^ ~km0);
+      const bool t1 = __builtin_amdgcn_inverse_ballot_w64(__ballot(o1 > k1[r]) ^ ~km1);
+      k0[r] = t0 ? o0 : k0[r];
+      k1[r] = t1 ? o1 : k1[r];
+    }
   }
-  bitonic128_desc<R>(e0, e1);
+}
+template <int SIZE, int STRIDE, int R>
+__device__ __forceinline__ void key_merge(uint32_t (&k0)[R], uint32_t (&k1)[R]) {
+  key_stage<SIZE, STRIDE, R>(k0, k1);
+  if constexpr (STRIDE > 1) key_merge<SIZE, STRIDE / 2, R>(k0, k1);
+}
+
+// Orders R 128-entry lists and writes the first k entries of each as fp32
+// values and int64 indices; a null values[r] skips the store of that row.  The
+// lists are left as they are; scratch[r] is 128 words of LDS owned by this wave.
+//
+// The network moves 32-bit words, half the work of moving entries: the upper 25
+// bits of the key with the entry's slot in the list below them.  The entries
+// are then fetched by slot, now in order except where neighbours agree in those
+// 25 bits; one in-lane and one cross-lane compare-exchange of whole entries
+// repair runs of two.  A final check of all neighbours sends the rare list
+// with a longer run through the full network on entries.  Equal values come
+// out by ascending index.
+// results are stored through pointers that name global memory (a generic
+// pointer would give flat stores)
+typedef float __attribute__((address_space(1))) * global_f32_out;
+typedef long long __attribute__((address_space(1))) * global_i64_out;
+
+template <int R>
+__device__ __forceinline__ void sort_and_store(const entry_t* const* list, uint32_t* const* scratch,
+                                               float* const* values, long long* const* indices,
+                                               int k) {
+  const int lane = threadIdx.x & 63;
+  uint32_t w0[R], w1[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    w0[r] = (entry_key(list[r][lane]) & ~0x7Fu) | lane;
+    w1[r] = (entry_key(list[r][lane + 64]) & ~0x7Fu) | (lane + 64);
+  }
+  key_merge<2, 1, R>(w0, w1);
+  key_merge<4, 2, R>(w0, w1);
+  key_merge<8, 4, R>(w0, w1);
+  key_merge<16, 8, R>(w0, w1);
+  key_merge<32, 16, R>(w0, w1);
+  key_merge<64, 32, R>(w0, w1);
+  key_merge<128, 64, R>(w0, w1);
+  // re-deal: lane l takes positions 2l and 2l+1, and fetches their entries
+  entry_t a[R], b[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    scratch[r][lane] = w0[r];
+    scratch[r][lane + 64] = w1[r];
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t sa = scratch[r][2 * lane], sb = scratch[r][2 * lane + 1];
+    a[r] = list[r][sa & 0x7Fu];
+    b[r] = list[r][sb & 0x7Fu];
+  }
+  const int up = ((lane + 1) & 63) << 2, down = ((lane + 63) & 63) << 2;
+  auto from = [&](int sel, entry_t v) {
+    return (static_cast<entry_t>(__builtin_amdgcn_ds_bpermute(sel, static_cast<uint32_t>(v >> 32))) << 32) |
+           static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(sel, static_cast<uint32_t>(v)));
+  };
+  bool bad = false;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    // positions (2l, 2l+1)
+    entry_t hi = a[r] > b[r] ? a[r] : b[r];
+    entry_t lo = a[r] > b[r] ? b[r] : a[r];
+    a[r] = hi;
+    b[r] = lo;
+    // positions (2l+1, 2l+2): b of this lane against a of the next
+    const entry_t na = from(up, a[r]);    // a of lane + 1
+    const entry_t pb = from(down, b[r]);  // b of lane - 1
+    const entry_t b2 = (lane < 63 && na > b[r]) ? na : b[r];
+    const entry_t a2 = (lane > 0 && a[r] > pb) ? pb : a[r];
+    a[r] = a2;
+    b[r] = b2;
+    // all neighbours in order?
+    const entry_t na2 = from(up, a[r]);
+    bad |= b[r] > a[r] || (lane < 63 && na2 > b[r]);
+  }
+  if (__ballot(bad) != 0ull) {
+    entry_t e0[R], e1[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      e0[r] = list[r][lane];
+      e1[r] = list[r][lane + 64];
+    }
+    bitonic128_desc<R>(e0, e1);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (!values[r]) continue;
+      global_f32_out gv = (global_f32_out)values[r];
+      global_i64_out gi = (global_i64_out)indices[r];
+      if (lane < k) {
+        gv[lane] = key2f(entry_key(e0[r]));
+        gi[lane] = entry_idx(e0[r]);
+      }
+      if (lane + 64 < k) {
+        gv[lane + 64] = key2f(entry_key(e1[r]));
+        gi[lane + 64] = entry_idx(e1[r]);
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (!values[r]) continue;
-    if (lane < k) {
-      values[r][lane] = key2f(entry_key(e0[r]));
-      indices[r][lane] = entry_idx(e0[r]);
+    global_f32_out gv = (global_f32_out)values[r];
+    global_i64_out gi = (global_i64_out)indices[r];
+    if (2 * lane < k) {
+      gv[2 * lane] = key2f(entry_key(a[r]));
+      gi[2 * lane] = entry_idx(a[r]);
     }
-    if (lane + 64 < k) {
-      values[r][lane + 64] = key2f(entry_key(e1[r]));
-      indices[r][lane + 64] = entry_idx(e1[r]);
+    if (2 * lane + 1 < k) {
+      gv[2 * lane + 1] = key2f(entry_key(b[r]));
+      gi[2 * lane + 1] = entry_idx(b[r]);
     }
   }
+}
+
+// sort_and_store<2> as a real function: its many mask constants and fragments
+// then live in the callee's registers only, instead of crowding the caller's
+// scalar registers for the whole kernel.  LDS pointers travel as such.
+typedef const entry_t __attribute__((address_space(3))) * lds_entry_ptr;
+typedef uint32_t __attribute__((address_space(3))) * lds_u32_ptr;
+__device__ __attribute__((noinline)) inline void sort_and_store_pair(lds_entry_ptr l0, lds_entry_ptr l1,
+                                                                     lds_u32_ptr scratch, float* v0,
+                                                                     float* v1, long long* i0,
+                                                                     long long* i1, int k) {
+  const entry_t* const lists[2] = {(const entry_t*)l0, (const entry_t*)l1};
+  uint32_t* const sc[2] = {(uint32_t*)scratch, (uint32_t*)scratch + kTop};
+  float* const cv[2] = {v0, v1};
+  long long* const ci[2] = {i0, i1};
+  sort_and_store<2>(lists, sc, cv, ci, k);
 }
 
 }  // namespace cmk

@@ -177,7 +177,6 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   for (int g = 0; g < kStripRows / kPassRows; ++g) {
     const int r0 = kPassRows * g + 2 * wave;
     if (a.splits == 1) {
-      const entry_t* const lists[2] = {list[r0], list[r0 + 1]};
       float* vals[2];
       long long* inds[2];
 #pragma unroll
@@ -187,9 +186,8 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
         vals[rr] = y < Yext ? a.values + orow * a.k : nullptr;
         inds[rr] = y < Yext ? a.indices + orow * a.k : nullptr;
       }
-      float* const cv[2] = {vals[0], vals[1]};
-      long long* const ci[2] = {inds[0], inds[1]};
-      sort_and_store<2>(lists, cv, ci, a.k);
+      sort_and_store_pair((lds_entry_ptr)list[r0], (lds_entry_ptr)list[r0 + 1], (lds_u32_ptr)cand,
+                          vals[0], vals[1], inds[0], inds[1], a.k);
     } else {
 #pragma unroll
       for (int rr = 0; rr < 2; ++rr) {
@@ -236,9 +234,10 @@ __global__ __launch_bounds__(kThreads) void topk_merge_kernel(const entry_t* par
     select128<18>(key, [&](int j) { return idx[j]; }, seed, cands[wave], list[wave]);
   }
   const entry_t* const lists[1] = {list[wave]};
+  uint32_t* const scratch[1] = {reinterpret_cast<uint32_t*>(cands[wave])};
   float* const cv[1] = {values + row * k};
   long long* const ci[1] = {indices + row * k};
-  sort_and_store<1>(lists, cv, ci, k);
+  sort_and_store<1>(lists, scratch, cv, ci, k);
 }
 
 // One wave per part of a 1-D array: keeps the best 128 of its range.
