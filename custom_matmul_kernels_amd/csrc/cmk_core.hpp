@@ -131,7 +131,7 @@ __device__ __forceinline__ void lane_offsets_bytes(const Operand& o,
 // running across slab and tile boundaries.  Inside a k-group all LDS traffic is
 // issued directly behind the group's first MFMA step, where it costs no
 // matrix-pipe time.
-template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32>
+template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32, bool APART = true>
 struct Core {
   static_assert(WX * WY == 4 || WX * WY == 8 || WX * WY == 16, "4, 8 or 16 waves per work-group");
   static constexpr int NT = WX * WY * 64;      // threads per work-group
@@ -153,6 +153,7 @@ struct Core {
   int lt, ls;                // (tile, slab) of the next slab to fetch (wave-uniform)
   int xbase, y0, K;
   int xr, yr, half;
+  int xrow[BX], yrow[BY];    // LDS row of each block; see begin()
   unsigned xoff[MX::NV];     // this lane's byte offsets for the direct loads
   unsigned yoff[MY::NV];
   float* pend_buf;           // buffer whose Y half is still to be requested (wave-uniform)
@@ -249,9 +250,9 @@ struct Core {
   __device__ __forceinline__ void read_frags(const float* buf, int kg, f32x4 (&fx)[BX],
                                              f32x4 (&fy)[BY]) {
 #pragma unroll
-    for (int b = 0; b < BX; ++b) fx[b] = frag<XK, TX>(buf, xr + 32 * b, kg);
+    for (int b = 0; b < BX; ++b) fx[b] = frag<XK, TX>(buf, xrow[b], kg);
 #pragma unroll
-    for (int b = 0; b < BY; ++b) fy[b] = frag<YK, TY>(buf + xFloats, yr + 32 * b, kg);
+    for (int b = 0; b < BY; ++b) fy[b] = frag<YK, TY>(buf + xFloats, yrow[b], kg);
   }
 
   // Waits until this wave's direct loads have landed in LDS.
@@ -268,6 +269,23 @@ struct Core {
     half = lane >> 5;
     xr = (wave % WX) * BX * 32 + (lane & 31);
     yr = (wave / WX) * BY * 32 + (lane & 31);
+    // The rows of a wave's blocks are 32 apart.  With APART the compiler is not
+    // told: it would fuse the 32-bit column reads of neighbouring blocks into
+    // two-address reads whose 8-bit offsets then need a vector add per pair, and
+    // vector instructions cost matrix-pipe time while LDS reads do not.  Kept
+    // apart, the reads of one block use immediate offsets from one address
+    // register, in pairs that share an LDS bank (measured: a gain for 128-row
+    // tiles, a loss for 256-row tiles).
+#pragma unroll
+    for (int b = 0; b < BX; ++b) {
+      xrow[b] = xr + 32 * b;
+      if (APART) asm volatile("" : "+v"(xrow[b]));
+    }
+#pragma unroll
+    for (int b = 0; b < BY; ++b) {
+      yrow[b] = yr + 32 * b;
+      if (APART) asm volatile("" : "+v"(yrow[b]));
+    }
     xbase = __builtin_amdgcn_readfirstlane(xbase_);
     y0 = __builtin_amdgcn_readfirstlane(y0_);
     K = __builtin_amdgcn_readfirstlane(K_);
