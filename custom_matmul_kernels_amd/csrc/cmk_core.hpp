@@ -131,7 +131,13 @@ __device__ __forceinline__ void lane_offsets_bytes(const Operand& o,
 // running across slab and tile boundaries.  Inside a k-group all LDS traffic is
 // issued directly behind the group's first MFMA step, where it costs no
 // matrix-pipe time.
-template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32, bool APART = true>
+// RC_READS picks how the four 32-bit column reads of a row-contiguous
+// operand's fragment are issued (vector adds cost matrix-pipe time, LDS reads
+// do not; which form wins was measured per tile shape):
+constexpr int kReadsPaired = 1;   // two-address reads (k, k+1) with immediate offsets, one bank each
+constexpr int kReadsSingle = 2;   // four single reads with immediate offsets
+
+template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32, int RC_READS = kReadsPaired>
 struct Core {
   static_assert(WX * WY == 4 || WX * WY == 8 || WX * WY == 16, "4, 8 or 16 waves per work-group");
   static constexpr int NT = WX * WY * 64;      // threads per work-group
@@ -169,13 +175,20 @@ struct Core {
                           ((long long)(T + KS) * o.ld < (1ll << 29));
     if (interior) {
       const long long first = KIND == KC ? (long long)r0 * o.ld + k0 : (long long)k0 * o.ld + r0;
-      const char* tile = reinterpret_cast<const char*>(o.p + first);
+      // the tile's address is the same in every lane; pinned to scalar registers
+      // so that each load is (scalar base + 32-bit lane offset) with no vector add
+      unsigned long long tile_bits = reinterpret_cast<unsigned long long>(o.p + first);
+      asm volatile("" : "+s"(tile_bits));
+      const char* tile = reinterpret_cast<const char*>(tile_bits);
       const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 #pragma unroll
       for (int p = 0; p < M::NV; ++p)
-        if (M::kEven || p * M::NW + wave < M::NI)
-          __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + off[p]),
+        if (M::kEven || p * M::NW + wave < M::NI) {
+          unsigned o32 = off[p];
+          asm volatile("" : "+v"(o32));  // keeps the offset a 32-bit register at this point
+          __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + o32),
                                            (lds_void_ptr)(dst + (p * M::NW + wave) * 256), 16, 0, 0);
+        }
     } else {
       // NT threads x 4 floats per pass, walking the tile in its memory order
       constexpr int RUN = KIND == KC ? KS : T;        // contiguous floats per line
@@ -237,8 +250,19 @@ struct Core {
     if constexpr (KIND == KC) {
       return *reinterpret_cast<const f32x4*>(&lds[lds_pos<KC, T, KS>(row, kg * 8 + half * 4)]);
     } else {
-      const float* q = &lds[(kg * 8 + half * 4) * T + row];
       f32x4 r;
+      if constexpr (RC_READS == kReadsSingle) {
+        // volatile keeps the reads single: 16-bit immediate offsets from one
+        // address register
+        const volatile float __attribute__((address_space(3)))* q =
+            (const volatile float __attribute__((address_space(3)))*)&lds[(kg * 8 + half * 4) * T + row];
+        r.x = q[0];
+        r.y = q[T];
+        r.z = q[2 * T];
+        r.w = q[3 * T];
+        return r;
+      }
+      const float* q = &lds[(kg * 8 + half * 4) * T + row];
       r.x = q[0];
       r.y = q[T];
       r.z = q[2 * T];
@@ -269,22 +293,20 @@ struct Core {
     half = lane >> 5;
     xr = (wave % WX) * BX * 32 + (lane & 31);
     yr = (wave / WX) * BY * 32 + (lane & 31);
-    // The rows of a wave's blocks are 32 apart.  With APART the compiler is not
-    // told: it would fuse the 32-bit column reads of neighbouring blocks into
-    // two-address reads whose 8-bit offsets then need a vector add per pair, and
-    // vector instructions cost matrix-pipe time while LDS reads do not.  Kept
-    // apart, the reads of one block use immediate offsets from one address
-    // register, in pairs that share an LDS bank (measured: a gain for 128-row
-    // tiles, a loss for 256-row tiles).
+    // The rows of a wave's blocks are 32 apart.  The compiler is not told: it
+    // would fuse the 32-bit column reads of neighbouring blocks into
+    // two-address reads whose 8-bit offsets then need a vector add per pair.
+    // Kept apart, the reads of one block pair up as (k, k+1) with immediate
+    // offsets from one address register.
 #pragma unroll
     for (int b = 0; b < BX; ++b) {
       xrow[b] = xr + 32 * b;
-      if (APART) asm volatile("" : "+v"(xrow[b]));
+      if (RC_READS == kReadsPaired) asm volatile("" : "+v"(xrow[b]));
     }
 #pragma unroll
     for (int b = 0; b < BY; ++b) {
       yrow[b] = yr + 32 * b;
-      if (APART) asm volatile("" : "+v"(yrow[b]));
+      if (RC_READS == kReadsPaired) asm volatile("" : "+v"(yrow[b]));
     }
     xbase = __builtin_amdgcn_readfirstlane(xbase_);
     y0 = __builtin_amdgcn_readfirstlane(y0_);
