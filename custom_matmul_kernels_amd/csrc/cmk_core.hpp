@@ -137,7 +137,8 @@ __device__ __forceinline__ void lane_offsets_bytes(const Operand& o,
 constexpr int kReadsPaired = 1;   // two-address reads (k, k+1) with immediate offsets, one bank each
 constexpr int kReadsSingle = 2;   // four single reads with immediate offsets
 
-template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32, int RC_READS = kReadsPaired>
+template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32, int RC_READS = kReadsPaired,
+          bool STAGGER = false>
 struct Core {
   static_assert(WX * WY == 4 || WX * WY == 8 || WX * WY == 16, "4, 8 or 16 waves per work-group");
   static constexpr int NT = WX * WY * 64;      // threads per work-group
@@ -164,6 +165,8 @@ struct Core {
   unsigned yoff[MY::NV];
   float* pend_buf;           // buffer whose Y half is still to be requested (wave-uniform)
   int pend_k0;
+  float* pend_xbuf;          // buffer whose X half is still to be requested (wave-uniform)
+  bool late;                 // this wave requests its slabs two k-groups after its SIMD partner
 
   // One operand's slab -> LDS.  Interior tiles: NV direct loads per wave.  Edge
   // tiles: every element is fetched from a clamped (always valid) address,
@@ -244,6 +247,10 @@ struct Core {
     if (pend_buf) fetch<YK, TY, MY>(Y, yoff, y0, pend_k0, pend_buf + xFloats);
     pend_buf = nullptr;
   }
+  __device__ __forceinline__ void issue_pending_x(const Operand& X) {
+    if (pend_xbuf) issue_x(X, pend_xbuf);
+    pend_xbuf = nullptr;
+  }
 
   template <int KIND, int T>
   __device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg) {
@@ -318,6 +325,12 @@ struct Core {
     it = 0;
     lt = 0;
     ls = 0;
+    pend_xbuf = nullptr;
+    // STAGGER: the upper half of the waves does its address arithmetic and load
+    // requests two k-groups after the lower half, which spreads the requests
+    // over the slab (measured: a gain for the 4-wave min kernel, a loss for the
+    // 8-wave top-k kernel)
+    late = STAGGER && __builtin_amdgcn_readfirstlane(wave) >= WX * WY / 2;
     issue_x(X, lds);
     issue_y(Y);
     wait_loads();
@@ -345,13 +358,16 @@ struct Core {
             acc[bx][by] = __builtin_amdgcn_mfma_f32_32x32x2f32(
                 xf[kg & 1][bx][0], yf[kg & 1][by][0], acc[bx][by], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (kg == 0) issue_y(Y);
+        if (kg == 0 && !late) issue_y(Y);
+        if (kg == 1 && late) issue_pending_x(X);
+        if (kg == 2 && late) issue_y(Y);
         if (kg + 1 < NG) {
           read_frags(cur, kg + 1, xf[(kg + 1) & 1], yf[(kg + 1) & 1]);
         } else if (has1) {
           wait_loads();     // this wave's part of slab it+1 is in LDS
           __syncthreads();  // everyone's is, and nobody reads `cur` any more
-          if (has2) issue_x(X, cur);
+          pend_xbuf = has2 ? cur : nullptr;
+          if (!late) issue_pending_x(X);
           read_frags(nxt, 0, xf[0], yf[0]);
         }
         __builtin_amdgcn_sched_barrier(0);

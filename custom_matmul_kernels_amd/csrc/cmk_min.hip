@@ -34,7 +34,7 @@ struct MinArgs {
 
 template <int XK, int YK>
 __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
-  using C = Core<XK, YK, 2, 2, 2, 2>;
+  using C = Core<XK, YK, 2, 2, 2, 2, 32, kReadsPaired, true>;
   __shared__ __attribute__((aligned(16))) float lds[C::ldsFloats];
 
   // Work-groups that are resident on one XCD at the same time form a block of
