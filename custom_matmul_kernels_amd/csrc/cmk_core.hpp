@@ -138,7 +138,7 @@ constexpr int kReadsPaired = 1;   // two-address reads (k, k+1) with immediate o
 constexpr int kReadsSingle = 2;   // four single reads with immediate offsets
 
 template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32, int RC_READS = kReadsPaired,
-          bool STAGGER = false>
+          bool STAGGER = false, bool Y_ONCE = false>
 struct Core {
   static_assert(WX * WY == 4 || WX * WY == 8 || WX * WY == 16, "4, 8 or 16 waves per work-group");
   static constexpr int NT = WX * WY * 64;      // threads per work-group
@@ -158,12 +158,15 @@ struct Core {
   f32x4 yf[2][BY];
   int it, iters, S;          // flat slab counter (wave-uniform)
   int lt, ls;                // (tile, slab) of the next slab to fetch (wave-uniform)
+  int ct, cs, nt;            // Y_ONCE: (tile, slab) being multiplied, tiles in the sequence
   int xbase, y0, K;
   int xr, yr, half;
+  int xfast, yfast;          // operand allows direct loads: aligned, offsets fit 32 bits (wave-uniform)
   int xrow[BX], yrow[BY];    // LDS row of each block; see begin()
   unsigned xoff[MX::NV];     // this lane's byte offsets for the direct loads
   unsigned yoff[MY::NV];
-  float* pend_buf;           // buffer whose Y half is still to be requested (wave-uniform)
+  float* pend_buf;           // where the Y slab that is still to be requested goes (wave-uniform)
+  float* ybase;              // Y_ONCE: the two Y buffers, behind the two X buffers
   int pend_k0;
   float* pend_xbuf;          // buffer whose X half is still to be requested (wave-uniform)
   bool late;                 // this wave requests its slabs two k-groups after its SIMD partner
@@ -173,9 +176,9 @@ struct Core {
   // zeroed when it lies outside the matrix, and stored from registers.
   template <int KIND, int T, class M>
   __device__ __forceinline__ void fetch(const Operand& o, const unsigned (&off)[M::NV], int r0,
-                                        int k0, float* dst) {
-    const bool interior = o.vec && (k0 + KS <= K) && (r0 + T <= o.rows) &&
-                          ((long long)(T + KS) * o.ld < (1ll << 29));
+                                        int k0, float* dst, int fast) {
+    // plain integers, so that the test stays in 32-bit scalar registers
+    const int interior = fast & static_cast<int>(k0 + KS <= K) & static_cast<int>(r0 + T <= o.rows);
     if (interior) {
       const long long first = KIND == KC ? (long long)r0 * o.ld + k0 : (long long)k0 * o.ld + r0;
       // the tile's address is the same in every lane; pinned to scalar registers
@@ -239,12 +242,18 @@ struct Core {
     // address arithmetic on the scalar unit
     const int x0 = __builtin_amdgcn_readfirstlane(xbase + lt * TX);
     pend_k0 = __builtin_amdgcn_readfirstlane(ls * KS);
-    pend_buf = buf;
-    fetch<XK, TX, MX>(X, xoff, x0, pend_k0, buf);
-    if (++ls == S) { ls = 0; ++lt; }
+    fetch<XK, TX, MX>(X, xoff, x0, pend_k0, buf, xfast);
+    if constexpr (Y_ONCE) {
+      // tiles run inside slabs: the Y slab is fetched with the first tile only
+      pend_buf = lt == 0 ? ybase + (ls & 1) * yFloats : nullptr;
+      if (++lt == nt) { lt = 0; ++ls; }
+    } else {
+      pend_buf = buf + xFloats;
+      if (++ls == S) { ls = 0; ++lt; }
+    }
   }
   __device__ __forceinline__ void issue_y(const Operand& Y) {
-    if (pend_buf) fetch<YK, TY, MY>(Y, yoff, y0, pend_k0, pend_buf + xFloats);
+    if (pend_buf) fetch<YK, TY, MY>(Y, yoff, y0, pend_k0, pend_buf, yfast);
     pend_buf = nullptr;
   }
   __device__ __forceinline__ void issue_pending_x(const Operand& X) {
@@ -278,12 +287,12 @@ struct Core {
     }
   }
   // Four k values (8*kg + 4*half + 0..3) of every block row of this lane.
-  __device__ __forceinline__ void read_frags(const float* buf, int kg, f32x4 (&fx)[BX],
-                                             f32x4 (&fy)[BY]) {
+  __device__ __forceinline__ void read_frags(const float* xb, const float* yb, int kg,
+                                             f32x4 (&fx)[BX], f32x4 (&fy)[BY]) {
 #pragma unroll
-    for (int b = 0; b < BX; ++b) fx[b] = frag<XK, TX>(buf, xrow[b], kg);
+    for (int b = 0; b < BX; ++b) fx[b] = frag<XK, TX>(xb, xrow[b], kg);
 #pragma unroll
-    for (int b = 0; b < BY; ++b) fy[b] = frag<YK, TY>(buf + xFloats, yrow[b], kg);
+    for (int b = 0; b < BY; ++b) fy[b] = frag<YK, TY>(yb, yrow[b], kg);
   }
 
   // Waits until this wave's direct loads have landed in LDS.
@@ -319,7 +328,13 @@ struct Core {
     y0 = __builtin_amdgcn_readfirstlane(y0_);
     K = __builtin_amdgcn_readfirstlane(K_);
     S = max(1, (K + KS - 1) / KS);
-    iters = __builtin_amdgcn_readfirstlane(ntiles) * S;
+    xfast = X.vec != 0 && (long long)(TX + KS) * X.ld < (1ll << 29);
+    yfast = Y.vec != 0 && (long long)(TY + KS) * Y.ld < (1ll << 29);
+    nt = __builtin_amdgcn_readfirstlane(ntiles);
+    iters = nt * S;
+    ct = 0;
+    cs = 0;
+    ybase = lds + 2 * xFloats;
     lane_offsets_bytes<XK, TX, KS, NT>(X, xoff);
     lane_offsets_bytes<YK, TY, KS, NT>(Y, yoff);
     it = 0;
@@ -335,16 +350,36 @@ struct Core {
     issue_y(Y);
     wait_loads();
     __syncthreads();
-    if (iters > 1) issue_x(X, lds + bufFloats);
-    read_frags(lds, 0, xf[0], yf[0]);
+    if (iters > 1) issue_x(X, xbuf(lds, 1));
+    read_frags(lds, ybuf(lds, 0, 0), 0, xf[0], yf[0]);
+  }
+
+  // LDS buffers of flat slab `i`, whose k-slab index is `s`.  Without Y_ONCE an
+  // X and a Y slab sit side by side, twice; with it, two X buffers are followed
+  // by two Y buffers that alternate with the k-slab.
+  __device__ __forceinline__ float* xbuf(float* lds, int i) const {
+    return lds + (i & 1) * (Y_ONCE ? xFloats : bufFloats);
+  }
+  __device__ __forceinline__ float* ybuf(float* lds, int i, int s) const {
+    return Y_ONCE ? lds + 2 * xFloats + (s & 1) * yFloats : xbuf(lds, i) + xFloats;
   }
 
   // acc += the current tile's product: S slabs of the flat sequence.
   __device__ __forceinline__ void tile(const Operand& X, const Operand& Y, float* lds,
                                        f32x16 (&acc)[BX][BY]) {
-    for (int s = 0; s < S; ++s) {
-      float* cur = lds + (it & 1) * bufFloats;
-      const float* nxt = lds + ((it + 1) & 1) * bufFloats;
+    static_assert(!Y_ONCE, "with Y_ONCE the kernel walks slabs itself: tiles inside k-slabs");
+    for (int s = 0; s < S; ++s) slab(X, Y, lds, acc);
+  }
+
+  // acc += one slab of the flat sequence.
+  __device__ __forceinline__ void slab(const Operand& X, const Operand& Y, float* lds,
+                                       f32x16 (&acc)[BX][BY]) {
+    {
+      float* cur = xbuf(lds, it);
+      const float* nxt = xbuf(lds, it + 1);
+      const int ns = (Y_ONCE && ct + 1 == nt) ? cs + 1 : cs;   // k-slab of the next flat slab
+      const float* ycur = ybuf(lds, it, cs);
+      const float* ynxt = ybuf(lds, it + 1, ns);
       const bool has1 = it + 1 < iters;
       const bool has2 = it + 2 < iters;
 #pragma unroll
@@ -362,13 +397,13 @@ struct Core {
         if (kg == 1 && late) issue_pending_x(X);
         if (kg == 2 && late) issue_y(Y);
         if (kg + 1 < NG) {
-          read_frags(cur, kg + 1, xf[(kg + 1) & 1], yf[(kg + 1) & 1]);
+          read_frags(cur, ycur, kg + 1, xf[(kg + 1) & 1], yf[(kg + 1) & 1]);
         } else if (has1) {
           wait_loads();     // this wave's part of slab it+1 is in LDS
           __syncthreads();  // everyone's is, and nobody reads `cur` any more
           pend_xbuf = has2 ? cur : nullptr;
           if (!late) issue_pending_x(X);
-          read_frags(nxt, 0, xf[0], yf[0]);
+          read_frags(nxt, ynxt, 0, xf[0], yf[0]);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -382,6 +417,7 @@ struct Core {
         __builtin_amdgcn_sched_barrier(0);
       }
       ++it;
+      if (Y_ONCE && ++ct == nt) { ct = 0; ++cs; }
     }
   }
 };

@@ -51,7 +51,7 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   // the two 32-row halves of the strip.  One work-group per CU; its two waves
   // per SIMD are always in the same phase, because on this part vector
   // instructions of one wave do not issue while another wave of the SIMD streams MFMAs.
-  using C = Core<XK, YK, 4, 2, 2, 1, 32, kReadsSingle>;
+  using C = Core<XK, YK, 4, 2, 2, 1, 32, kReadsSingle, false, true>;
   static_assert(C::TX == kTileX && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
   constexpr int stageFloats = kPassRows * kStagePitch;
   constexpr int bandFloats = 8 * kCand * 2;  // one candidate list per wave
@@ -111,10 +111,15 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
     core.begin(X, Y, xt0 * C::TX, y0, a.K, nt, lds);
     f32x16 acc[kChunkTiles][2][1];
 #pragma unroll
-    for (int i = 0; i < kChunkTiles; ++i) {
+    for (int i = 0; i < kChunkTiles; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][0][0][r] = acc[i][1][0][r] = 0.f;
-      if (i < nt) core.tile(X, Y, lds, acc[i]);
+    // k-slabs outside, tiles inside: a slab of the strip's own rows is fetched
+    // once and meets the chunk's tiles one after the other
+    for (int s = 0; s < core.S; ++s) {
+#pragma unroll
+      for (int i = 0; i < kChunkTiles; ++i)
+        if (i < nt) core.slab(X, Y, lds, acc[i]);
     }
     __syncthreads();  // all fragment reads are done; the buffers become the staging area
 
