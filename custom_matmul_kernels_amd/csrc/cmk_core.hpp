@@ -159,6 +159,9 @@ struct Core {
   int it, iters, S;          // flat slab counter (wave-uniform)
   int lt, ls;                // (tile, slab) of the next slab to fetch (wave-uniform)
   int ct, cs, nt;            // Y_ONCE: (tile, slab) being multiplied, tiles in the sequence
+  // element offset of the next slab to fetch within each operand, advanced by
+  // additions from slab to slab (all wave-uniform)
+  long long xrun, yrun, xstep_in, xstep_out, ystep;
   int xbase, y0, K;
   int xr, yr, half;
   int xfast, yfast;          // operand allows direct loads: aligned, offsets fit 32 bits (wave-uniform)
@@ -168,6 +171,7 @@ struct Core {
   float* pend_buf;           // where the Y slab that is still to be requested goes (wave-uniform)
   float* ybase;              // Y_ONCE: the two Y buffers, behind the two X buffers
   int pend_k0;
+  long long pend_y;          // and its element offset
   float* pend_xbuf;          // buffer whose X half is still to be requested (wave-uniform)
   bool late;                 // this wave requests its slabs two k-groups after its SIMD partner
 
@@ -176,11 +180,10 @@ struct Core {
   // zeroed when it lies outside the matrix, and stored from registers.
   template <int KIND, int T, class M>
   __device__ __forceinline__ void fetch(const Operand& o, const unsigned (&off)[M::NV], int r0,
-                                        int k0, float* dst, int fast) {
+                                        int k0, long long first, float* dst, int fast) {
     // plain integers, so that the test stays in 32-bit scalar registers
     const int interior = fast & static_cast<int>(k0 + KS <= K) & static_cast<int>(r0 + T <= o.rows);
     if (interior) {
-      const long long first = KIND == KC ? (long long)r0 * o.ld + k0 : (long long)k0 * o.ld + r0;
       // the tile's address is the same in every lane; pinned to scalar registers
       // so that each load is (scalar base + 32-bit lane offset) with no vector add
       unsigned long long tile_bits = reinterpret_cast<unsigned long long>(o.p + first);
@@ -242,18 +245,23 @@ struct Core {
     // address arithmetic on the scalar unit
     const int x0 = __builtin_amdgcn_readfirstlane(xbase + lt * TX);
     pend_k0 = __builtin_amdgcn_readfirstlane(ls * KS);
-    fetch<XK, TX, MX>(X, xoff, x0, pend_k0, buf, xfast);
+    fetch<XK, TX, MX>(X, xoff, x0, pend_k0, xrun, buf, xfast);
     if constexpr (Y_ONCE) {
       // tiles run inside slabs: the Y slab is fetched with the first tile only
       pend_buf = lt == 0 ? ybase + (ls & 1) * yFloats : nullptr;
-      if (++lt == nt) { lt = 0; ++ls; }
+      pend_y = yrun;
+      xrun += xstep_in;
+      if (++lt == nt) { lt = 0; ++ls; xrun += xstep_out; yrun += ystep; }
     } else {
       pend_buf = buf + xFloats;
-      if (++ls == S) { ls = 0; ++lt; }
+      pend_y = yrun;
+      xrun += xstep_in;
+      yrun += ystep;
+      if (++ls == S) { ls = 0; ++lt; xrun += xstep_out; yrun -= S * ystep; }
     }
   }
   __device__ __forceinline__ void issue_y(const Operand& Y) {
-    if (pend_buf) fetch<YK, TY, MY>(Y, yoff, y0, pend_k0, pend_buf, yfast);
+    if (pend_buf) fetch<YK, TY, MY>(Y, yoff, y0, pend_k0, pend_y, pend_buf, yfast);
     pend_buf = nullptr;
   }
   __device__ __forceinline__ void issue_pending_x(const Operand& X) {
@@ -334,6 +342,17 @@ struct Core {
     iters = nt * S;
     ct = 0;
     cs = 0;
+    {
+      // steps of the running offsets: to the next slab of the inner loop, and
+      // the correction when the inner loop wraps
+      const long long xs_tile = XK == KC ? (long long)TX * X.ld : TX;
+      const long long xs_slab = XK == KC ? KS : (long long)KS * X.ld;
+      xrun = XK == KC ? (long long)xbase * X.ld : xbase;
+      yrun = YK == KC ? (long long)y0 * Y.ld : y0;
+      ystep = YK == KC ? KS : (long long)KS * Y.ld;
+      if (Y_ONCE) { xstep_in = xs_tile; xstep_out = xs_slab - nt * xs_tile; }
+      else        { xstep_in = xs_slab; xstep_out = xs_tile - S * xs_slab; }
+    }
     ybase = lds + 2 * xFloats;
     lane_offsets_bytes<XK, TX, KS, NT>(X, xoff);
     lane_offsets_bytes<YK, TY, KS, NT>(Y, yoff);
