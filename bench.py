@@ -28,8 +28,8 @@ PEAK_HBM_GBS = 8000.0
 # traffic = (2 * FETCH_SIZE + WRITE_SIZE) * 1024.  The counters cannot be read
 # from inside this process; the figures are those of the summaries in profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "min_bmm_large": (2 * 1.52705e6 + 2048) * 1024,      # profiles/min_kernel_min_bmm_large.txt
-    "topk_bmm": (2 * 575644 + 1.57286e6) * 1024,          # profiles/topk_kernel_topk_bmm.txt
+    "min_bmm_large": (2 * 2.13965e6 + 2048) * 1024,      # profiles/min_kernel_min_bmm_large.txt
+    "topk_bmm": (2 * 785073 + 1.57286e6) * 1024,          # profiles/topk_kernel_topk_bmm.txt
 }
 
 
@@ -161,8 +161,9 @@ def cpu_baseline(torch, wl, args_dev, budget_s=12.0):
     gflops = done_rows * wl["cpu_flop_per_row"] / t_total / 1e9
     return {"value": round(gflops, 2), "unit": "GFLOP/s", "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": "%s on %d of %d rows, %d threads, %.2f s" % (
-                wl["cpu_expr"], done_rows, wl["rows"], torch.get_num_threads(), t_total)}
+            "sample": "%s on %d rows in slabs of %d (%.2f passes over the workload's %d rows), "
+                      "%d threads, %.2f s" % (wl["cpu_expr"], done_rows, rows, done_rows / wl["rows"],
+                                              wl["rows"], torch.get_num_threads(), t_total)}
 
 
 def run_workload(torch, wl, steps, warmup):
