@@ -24,6 +24,9 @@ struct BmmArgs {
   int vecA, vecB;
 };
 
+constexpr int kMaskRows = 128;    // element-mask tile staged in LDS: rows ...
+constexpr int kMaskPitch = 144;   // ... of 128 bytes, 16-byte aligned, skewed over the banks
+
 template <int XK, int YK, bool MASKED>
 __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
   using C = Core<XK, YK, 2, 2, 2, 2>;
@@ -92,6 +95,37 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     core.tile(X, Y, lds, acc);
 
+    // A kept tile whose masks can be fetched with 16-byte loads gets them staged
+    // in LDS (the operand buffers are free by now): 128 rows of 128 element-mask
+    // bytes, then the tile's 16x16 thread-mask bytes.
+    bool staged = false;
+    if constexpr (MASKED) {
+      const int m0 = (tile_m0 + ti) * C::TX;
+      staged = m0 + 128 <= a.M && n0 + 128 <= a.N && (a.N & 15) == 0 &&
+               (reinterpret_cast<uintptr_t>(a.element_mask) & 15) == 0;
+      if (staged) {
+        typedef const f32x4 __attribute__((address_space(1))) * g16p;
+        typedef const uint8_t __attribute__((address_space(1))) * g1p;
+        core.wait_loads();
+        __syncthreads();  // nobody reads operand fragments any more
+        uint8_t* ml = reinterpret_cast<uint8_t*>(lds);
+        const uint8_t* eb = a.element_mask + (mb * a.M + m0) * a.N + n0;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          const int idx = threadIdx.x + kThreads * p;
+          const int row = idx >> 3, c16 = (idx & 7) * 16;
+          const f32x4 v = *(g16p)(eb + (long long)row * a.N + c16);
+          *reinterpret_cast<f32x4*>(ml + row * kMaskPitch + c16) = v;
+        }
+        const int tn8 = (a.N + 7) >> 3;
+        const int tm8 = (a.M + 7) >> 3;
+        ml[kMaskRows * kMaskPitch + threadIdx.x] =
+            *(g1p)(a.thread_mask + (mb * tm8 + (m0 >> 3) + (threadIdx.x >> 4)) * tn8 + (n0 >> 3) +
+                   (threadIdx.x & 15));
+        __syncthreads();
+      }
+    }
+
     // store: one accumulator register covers two 128-byte row segments of C
     const int wv = __builtin_amdgcn_readfirstlane(wave);
     const int mw = (tile_m0 + ti) * C::TX + (wv % 2) * 64;
@@ -110,6 +144,31 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
             char* rp = base + (long long)(bx * 32 + 8 * (r >> 2) + (r & 3)) * a.N * 4;
 #pragma unroll
             for (int by = 0; by < 2; ++by) *(gfp)(rp + voff + by * 128) = acc[bx][by][r];
+          }
+      } else if (staged) {
+        // masks come from LDS: byte reads there cost no vector-memory instructions
+        const uint8_t* ml = reinterpret_cast<const uint8_t*>(lds);
+        const int mwl = (wv % 2) * 64, nwl = (wv / 2) * 64;
+        const uint8_t* tl = ml + kMaskRows * kMaskPitch + (mwl >> 3) * 16 + (nwl >> 3) + (l32 >> 3);
+        const uint8_t* el = ml + (mwl + 4 * half) * kMaskPitch + nwl + l32;
+#pragma unroll
+        for (int bx = 0; bx < 2; ++bx)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            uint8_t tmk[2];
+#pragma unroll
+            for (int by = 0; by < 2; ++by) tmk[by] = tl[(bx * 4 + q) * 16 + by * 4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int r = 4 * q + e;
+              const int rowc = bx * 32 + 8 * q + e;
+              char* rp = base + (long long)rowc * a.N * 4;
+#pragma unroll
+              for (int by = 0; by < 2; ++by) {
+                const uint8_t em = el[rowc * kMaskPitch + by * 32];
+                *(gfp)(rp + voff + by * 128) = tmk[by] ? acc[bx][by][r] * (float)em : 0.f;
+              }
+            }
           }
       } else {
         const int tn8 = (a.N + 7) >> 3;

@@ -133,6 +133,22 @@ def test_mbmm_mask_precedence_and_integer_exactness(device):
     want = torch.from_numpy(O.c_mbmm(A.numpy(), B.numpy(), bm.numpy(), tm.numpy(), em.numpy(), False))
     O.check_values(C, want, 8)
     assert (C[0, 128:, :128] == 0).all() and (C[0, :8, 8:16] == 0).all() and C[0, 20, 30] == 0
+    # the same on a shape whose kept tiles take their masks through LDS (N % 16 == 0)
+    A2, B2 = seeded(1, 256, 256, 8, seed=8)
+    bm2 = torch.ones(1, 2, 2, dtype=torch.uint8)
+    tm2 = torch.ones(1, 32, 32, dtype=torch.uint8)
+    em2 = torch.ones(1, 256, 256, dtype=torch.uint8)
+    bm2[0, 1, 0] = 0
+    tm2[0, 0, 1] = 0
+    tm2[0, 31, 31] = 0
+    em2[0, 20, 30] = 0
+    em2[0, 21, 31] = 3
+    em2[0, 200, 250] = 7
+    C2 = MBMMCUDA()(A2.to(device), B2.to(device), bm2.to(device), tm2.to(device), em2.to(device)).cpu()
+    want2 = torch.from_numpy(O.c_mbmm(A2.numpy(), B2.numpy(), bm2.numpy(), tm2.numpy(), em2.numpy(), False))
+    O.check_values(C2, want2, 8)
+    assert (C2[0, 128:, :128] == 0).all() and (C2[0, :8, 8:16] == 0).all() and C2[0, 20, 30] == 0
+    assert (C2[0, 248:, 248:] == 0).all()
     # all-ones masks reproduce bmm, an all-zero block mask gives zeros
     ones = [torch.ones_like(t).to(device) for t in (bm, tm, em)]
     assert torch.equal(MBMMCUDA()(A.to(device), B.to(device), *ones), BMMCUDA()(A.to(device), B.to(device)))
