@@ -2,8 +2,8 @@
 // one axis; the product never reaches HBM.
 //
 // X = the reduced axis (inside a lane), Y = the kept axis.  A work-group of
-// eight waves owns a strip of 64 complete output rows and walks the reduced
-// axis in chunks of 1024 candidates (8 tiles of 128) whose accumulators all
+// sixteen waves owns a strip of 64 complete output rows and walks the reduced
+// axis in chunks of 1024 candidates (4 tiles of 256) whose accumulators all
 // stay in registers.  After each chunk the accumulators go through LDS, sixteen
 // rows at a time, so that one wave sees one row's 1024 candidates (16 per lane)
 // together with the row's running list (2 per lane); select128() keeps the best
@@ -36,40 +36,44 @@ struct TopkArgs {
   int ystrips, xtiles, splits, tiles_per_split;
 };
 
-constexpr int kTopkThreads = 512;
+constexpr int kTopkThreads = 1024;
 constexpr int kStripRows = 64;    // output rows per work-group
 constexpr int kPassRows = 16;     // rows staged through LDS per selection pass
 
-// MULTI = false: the whole reduced axis is one chunk (at most 1024 candidates).
-// The running lists are then only written after the product is finished, so
-// they may share LDS with the operand buffers, which leaves room for slabs of
-// depth 64 (half as many barriers per MFMA).  MULTI = true keeps the lists
-// apart and uses slabs of depth 32.
+// MULTI = false: the whole reduced axis is one chunk (at most 1024 candidates);
+// the lists are then only written after the product is finished and may share
+// LDS with the operand buffers.  MULTI = true: the lists carry state from chunk
+// to chunk and sit behind the operand buffers.
 template <int XK, int YK, bool MULTI>
 __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
-  // eight waves: wave % 4 picks 32 of a tile's 128 candidates, wave / 4 one of
-  // the two 32-row halves of the strip.  One work-group per CU; its two waves
-  // per SIMD are always in the same phase, because on this part vector
-  // instructions of one wave do not issue while another wave of the SIMD streams MFMAs.
-  using C = Core<XK, YK, 4, 2, 2, 1, 32, kReadsSingle, false, true>;
+  // Sixteen waves, four per SIMD: selection and ordering are long chains of
+  // dependent vector, scalar and LDS instructions, of which one wave issues one
+  // every 5 to 10 cycles; four waves keep the SIMD's issue slots far better
+  // filled than two (measured: 1.4x).  The phases of a work-group cannot
+  // overlap on this part (vector instructions of one wave do not issue while
+  // another wave of the SIMD streams MFMAs): all waves multiply, then all select.
+  // wave % 8 picks 32 of a tile's 256 candidates, wave / 8 one of the two 32-row
+  // halves of the strip; a wave's 64 accumulator registers cover 4 tiles =
+  // 1024 candidates x 32 rows.
+  using C = Core<XK, YK, 8, 2, 1, 1, 32, kReadsSingle, false, true>;
   static_assert(C::TX == kTileX && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
   constexpr int stageFloats = kPassRows * kStagePitch;
-  constexpr int bandFloats = 8 * kCand * 2;  // one candidate list per wave
+  constexpr int frontFloats = C::ldsFloats > stageFloats ? C::ldsFloats : stageFloats;
   constexpr int listFloats = kStripRows * kTop * 2;
-  constexpr int selFloats = stageFloats + bandFloats + listFloats;
-  static_assert(C::ldsFloats <= (MULTI ? stageFloats + bandFloats : selFloats),
-                "operand buffers must not reach the lists when these carry state between chunks");
+  constexpr int selFloats = frontFloats + listFloats;
+  static_assert(selFloats * 4 <= 160 * 1024, "LDS capacity");
   __shared__ __attribute__((aligned(16))) float lds[selFloats];
   // running top-128 of every row of the strip
-  entry_t(*list)[kTop] = reinterpret_cast<entry_t(*)[kTop]>(lds + stageFloats + bandFloats);
+  entry_t(*list)[kTop] = reinterpret_cast<entry_t(*)[kTop]>(lds + frontFloats);
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int l32 = lane & 31;
   const int half = lane >> 5;
-  const int wx = wave & 3;   // which 32 candidates of a tile
-  const int wy = wave >> 2;  // which half of the strip's rows
-  entry_t* cand = reinterpret_cast<entry_t*>(lds + stageFloats) + wave * kCand;
+  const int wx = wave & 7;   // which 32 candidates of a tile
+  const int wy = wave >> 3;  // which half of the strip's rows
+  // a staged row, once in registers, lends its space to the candidate list
+  entry_t* cand = reinterpret_cast<entry_t*>(lds + wave * kStagePitch);
   // the previous row's threshold seeds the next search; it carries over from
   // strip to strip, since neighbouring strips are statistically alike
   uint32_t seed = 0u;
@@ -109,11 +113,11 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
     const int nt = min(kChunkTiles, xt_end - xt0);
     __syncthreads();  // previous chunk's staging reads are finished
     core.begin(X, Y, xt0 * C::TX, y0, a.K, nt, lds);
-    f32x16 acc[kChunkTiles][2][1];
+    f32x16 acc[kChunkTiles][1][1];
 #pragma unroll
     for (int i = 0; i < kChunkTiles; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][0][0][r] = acc[i][1][0][r] = 0.f;
+      for (int r = 0; r < 16; ++r) acc[i][0][0][r] = 0.f;
     // k-slabs outside, tiles inside: a slab of the strip's own rows is fetched
     // once and meets the chunk's tiles one after the other
     for (int s = 0; s < core.S; ++s) {
@@ -130,22 +134,20 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
       if (g) __syncthreads();  // previous pass has been read
       // rows 16g .. 16g+15 live in the waves with wy == g / 2, lanes l32 / 16 == g % 2
       if (wy == (g >> 1) && (l32 >> 4) == (g & 1)) {
-        float* row = lds + (l32 & 15) * kStagePitch + wx * 64 + 4 * half;
+        float* row = lds + (l32 & 15) * kStagePitch + wx * 32 + 4 * half;
 #pragma unroll
         for (int i = 0; i < kChunkTiles; ++i)
 #pragma unroll
-          for (int bx = 0; bx < 2; ++bx)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              f32x4 v = {acc[i][bx][0][4 * q], acc[i][bx][0][4 * q + 1], acc[i][bx][0][4 * q + 2],
-                         acc[i][bx][0][4 * q + 3]};
-              *reinterpret_cast<f32x4*>(row + i * kTileX + bx * 32 + 8 * q) = v;
-            }
+          for (int q = 0; q < 4; ++q) {
+            f32x4 v = {acc[i][0][0][4 * q], acc[i][0][0][4 * q + 1], acc[i][0][0][4 * q + 2],
+                       acc[i][0][0][4 * q + 3]};
+            *reinterpret_cast<f32x4*>(row + i * kTileX + 8 * q) = v;
+          }
       }
       __syncthreads();
 #pragma unroll 1
-      for (int rr = 0; rr < 2; ++rr) {
-        const int pr = 2 * wave + rr;          // row of the pass, owned by this wave
+      for (int rr = 0; rr < 1; ++rr) {
+        const int pr = wave;                   // row of the pass, owned by this wave
         const int r = kPassRows * g + pr;      // row of the strip
         if (y0 + r >= Yext) continue;
         const float* src = lds + pr * kStagePitch;
@@ -177,30 +179,31 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
     }
   }
 
-  // each wave finishes the rows it owns, two at a time
+  // each wave finishes the four rows it owns, two at a time
 #pragma unroll 1
-  for (int g = 0; g < kStripRows / kPassRows; ++g) {
-    const int r0 = kPassRows * g + 2 * wave;
+  for (int g = 0; g < 4; g += 2) {
+    const int ra = kPassRows * g + wave, rb = ra + kPassRows;
     if (a.splits == 1) {
       float* vals[2];
       long long* inds[2];
 #pragma unroll
       for (int rr = 0; rr < 2; ++rr) {
-        const int y = y0 + r0 + rr;
+        const int y = y0 + (rr ? rb : ra);
         const long long orow = (long long)b * Yext + y;
         vals[rr] = y < Yext ? a.values + orow * a.k : nullptr;
         inds[rr] = y < Yext ? a.indices + orow * a.k : nullptr;
       }
-      sort_and_store_pair((lds_entry_ptr)list[r0], (lds_entry_ptr)list[r0 + 1], (lds_u32_ptr)cand,
+      sort_and_store_pair((lds_entry_ptr)list[ra], (lds_entry_ptr)list[rb], (lds_u32_ptr)cand,
                           vals[0], vals[1], inds[0], inds[1], a.k);
     } else {
 #pragma unroll
       for (int rr = 0; rr < 2; ++rr) {
-        const int y = y0 + r0 + rr;
+        const int r = rr ? rb : ra;
+        const int y = y0 + r;
         if (y >= Yext) continue;
         const long long o = ((long long)split * a.L * Yext + (long long)b * Yext + y) * kTop;
-        a.part[o + lane] = list[r0 + rr][lane];
-        a.part[o + lane + 64] = list[r0 + rr][lane + 64];
+        a.part[o + lane] = list[r][lane];
+        a.part[o + lane + 64] = list[r][lane + 64];
       }
     }
   }
