@@ -57,14 +57,16 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   // 1024 candidates x 32 rows.
   using C = Core<XK, YK, 8, 2, 1, 1, 32, kReadsSingle, false, true>;
   static_assert(C::TX == kTileX && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
+  // LDS: operand buffers, reused as the staging area; the lists follow the
+  // staging area (MULTI: the operand buffers, which they must outlive)
   constexpr int stageFloats = kPassRows * kStagePitch;
-  constexpr int frontFloats = C::ldsFloats > stageFloats ? C::ldsFloats : stageFloats;
   constexpr int listFloats = kStripRows * kTop * 2;
-  constexpr int selFloats = frontFloats + listFloats;
+  constexpr int listAt = MULTI ? (C::ldsFloats > stageFloats ? C::ldsFloats : stageFloats) : stageFloats;
+  constexpr int selFloats = listAt + listFloats > C::ldsFloats ? listAt + listFloats : C::ldsFloats;
   static_assert(selFloats * 4 <= 160 * 1024, "LDS capacity");
   __shared__ __attribute__((aligned(16))) float lds[selFloats];
   // running top-128 of every row of the strip
-  entry_t(*list)[kTop] = reinterpret_cast<entry_t(*)[kTop]>(lds + frontFloats);
+  entry_t(*list)[kTop] = reinterpret_cast<entry_t(*)[kTop]>(lds + listAt);
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
