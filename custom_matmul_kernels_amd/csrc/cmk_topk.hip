@@ -55,8 +55,15 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   // wave % 8 picks 32 of a tile's 256 candidates, wave / 8 one of the two 32-row
   // halves of the strip; a wave's 64 accumulator registers cover 4 tiles =
   // 1024 candidates x 32 rows.
-  using C = Core<XK, YK, 8, 2, 1, 1, 32, kReadsSingle, false, true>;
-  static_assert(C::TX == kTileX && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
+  // With a single chunk the operand buffers may fill LDS (the lists are written
+  // after the product), which allows tiles of 512 candidates, two 32x32 blocks
+  // per wave: half as many fragment reads of the strip's rows and half as many
+  // barriers per MFMA.
+  constexpr int kBX = MULTI ? 1 : 2;
+  constexpr int kTX = kTileX * kBX;             // candidates per tile in this kernel
+  constexpr int kCT = kChunkTiles / kBX;        // tiles per chunk in this kernel
+  using C = Core<XK, YK, 8, 2, kBX, 1, 32, kReadsSingle, false, true>;
+  static_assert(C::TX == kTX && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
   // LDS: operand buffers, reused as the staging area; the lists follow the
   // staging area (MULTI: the operand buffers, which they must outlive)
   constexpr int stageFloats = kPassRows * kStagePitch;
@@ -101,7 +108,7 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   Operand X = a.X, Y = a.Y;
   X.p = uniform_ptr(X.p + (long long)b * a.strideX);
   Y.p = uniform_ptr(Y.p + (long long)b * a.strideY);
-  const int x_limit = min(X.rows, xt_end * C::TX);
+  const int x_limit = min(X.rows, xt_end * kTileX);
   const int Yext = Y.rows;
 
   if constexpr (MULTI) {
@@ -112,39 +119,43 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   C core;
 
   for (int xt0 = xt_begin; xt0 < xt_end; xt0 += kChunkTiles) {
-    const int nt = min(kChunkTiles, xt_end - xt0);
+    const int nt = (min(kChunkTiles, xt_end - xt0) + kBX - 1) / kBX;
     __syncthreads();  // previous chunk's staging reads are finished
-    core.begin(X, Y, xt0 * C::TX, y0, a.K, nt, lds);
-    f32x16 acc[kChunkTiles][1][1];
+    core.begin(X, Y, xt0 * kTileX, y0, a.K, nt, lds);
+    f32x16 acc[kCT][kBX][1];
 #pragma unroll
-    for (int i = 0; i < kChunkTiles; ++i)
+    for (int i = 0; i < kCT; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][0][0][r] = 0.f;
+      for (int bx = 0; bx < kBX; ++bx)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][bx][0][r] = 0.f;
     // k-slabs outside, tiles inside: a slab of the strip's own rows is fetched
     // once and meets the chunk's tiles one after the other
     for (int s = 0; s < core.S; ++s) {
 #pragma unroll
-      for (int i = 0; i < kChunkTiles; ++i)
+      for (int i = 0; i < kCT; ++i)
         if (i < nt) core.slab(X, Y, lds, acc[i]);
     }
     __syncthreads();  // all fragment reads are done; the buffers become the staging area
 
     // selection, sixteen rows of the strip per pass
-    const int xc0 = xt0 * C::TX;
+    const int xc0 = xt0 * kTileX;
 #pragma unroll 1
     for (int g = 0; g < kStripRows / kPassRows; ++g) {
       if (g) __syncthreads();  // previous pass has been read
       // rows 16g .. 16g+15 live in the waves with wy == g / 2, lanes l32 / 16 == g % 2
       if (wy == (g >> 1) && (l32 >> 4) == (g & 1)) {
-        float* row = lds + (l32 & 15) * kStagePitch + wx * 32 + 4 * half;
+        float* row = lds + (l32 & 15) * kStagePitch + wx * 32 * kBX + 4 * half;
 #pragma unroll
-        for (int i = 0; i < kChunkTiles; ++i)
+        for (int i = 0; i < kCT; ++i)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            f32x4 v = {acc[i][0][0][4 * q], acc[i][0][0][4 * q + 1], acc[i][0][0][4 * q + 2],
-                       acc[i][0][0][4 * q + 3]};
-            *reinterpret_cast<f32x4*>(row + i * kTileX + 8 * q) = v;
-          }
+          for (int bx = 0; bx < kBX; ++bx)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              f32x4 v = {acc[i][bx][0][4 * q], acc[i][bx][0][4 * q + 1], acc[i][bx][0][4 * q + 2],
+                         acc[i][bx][0][4 * q + 3]};
+              *reinterpret_cast<f32x4*>(row + i * kTX + bx * 32 + 8 * q) = v;
+            }
       }
       __syncthreads();
 #pragma unroll 1
