@@ -96,11 +96,11 @@ struct LoadMap {
 // Byte offset, relative to the tile's first element in global memory, of the 16
 // bytes this lane fetches with its p-th direct load.
 template <int KIND, int T, int KS, int NT>
-__device__ __forceinline__ void lane_offsets_bytes(const Operand& o,
+__device__ __forceinline__ void lane_offsets_bytes(const Operand& o, int tid,
                                                    unsigned (&off)[LoadMap<KIND, T, KS, NT>::NV]) {
   using M = LoadMap<KIND, T, KS, NT>;
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
 #pragma unroll
   for (int p = 0; p < M::NV; ++p) {
     const int q = p * M::NW + wave;
@@ -163,7 +163,7 @@ struct Core {
   // additions from slab to slab (all wave-uniform)
   long long xrun, yrun, xstep_in, xstep_out, ystep;
   int xbase, y0, K;
-  int xr, yr, half;
+  int xr, yr, half, tid;
   int xfast, yfast;          // operand allows direct loads: aligned, offsets fit 32 bits (wave-uniform)
   int xrow[BX], yrow[BY];    // LDS row of each block; see begin()
   unsigned xoff[MX::NV];     // this lane's byte offsets for the direct loads
@@ -189,7 +189,7 @@ struct Core {
       unsigned long long tile_bits = reinterpret_cast<unsigned long long>(o.p + first);
       asm volatile("" : "+s"(tile_bits));
       const char* tile = reinterpret_cast<const char*>(tile_bits);
-      const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+      const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 #pragma unroll
       for (int p = 0; p < M::NV; ++p)
         if (M::kEven || p * M::NW + wave < M::NI) {
@@ -206,7 +206,7 @@ struct Core {
       constexpr int LINES = KIND == KC ? T : KS;
       constexpr int PASSES = (LINES + LPP - 1) / LPP;
       constexpr bool kAllLines = PASSES * LPP == LINES;  // otherwise some threads have no line
-      const int t = threadIdx.x;
+      const int t = tid;
       const int c4 = (t % TPR) * 4;
       f32x4 v[PASSES];
       const bool any = K > 0 && o.rows > 0;
@@ -312,8 +312,13 @@ struct Core {
   // slab 1 in flight.  Ends with every wave past a barrier.
   __device__ __forceinline__ void begin(const Operand& X, const Operand& Y, int xbase_, int y0_,
                                         int K_, int ntiles, float* lds) {
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    // The thread id is made opaque per sequence: values derived from it are
+    // then computed where they are used instead of being hoisted out of a
+    // kernel's outer loops, where they would only occupy (or spill) registers.
+    tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
     half = lane >> 5;
     xr = (wave % WX) * BX * 32 + (lane & 31);
     yr = (wave / WX) * BY * 32 + (lane & 31);
@@ -354,8 +359,8 @@ struct Core {
       else        { xstep_in = xs_slab; xstep_out = xs_tile - S * xs_slab; }
     }
     ybase = lds + 2 * xFloats;
-    lane_offsets_bytes<XK, TX, KS, NT>(X, xoff);
-    lane_offsets_bytes<YK, TY, KS, NT>(Y, yoff);
+    lane_offsets_bytes<XK, TX, KS, NT>(X, tid, xoff);
+    lane_offsets_bytes<YK, TY, KS, NT>(Y, tid, yoff);
     it = 0;
     lt = 0;
     ls = 0;

@@ -75,14 +75,7 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   // running top-128 of every row of the strip
   entry_t(*list)[kTop] = reinterpret_cast<entry_t(*)[kTop]>(lds + listAt);
 
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int l32 = lane & 31;
-  const int half = lane >> 5;
-  const int wx = wave & 7;   // which 32 candidates of a tile
-  const int wy = wave >> 3;  // which half of the strip's rows
-  // a staged row, once in registers, lends its space to the candidate list
-  entry_t* cand = reinterpret_cast<entry_t*>(lds + wave * kStagePitch);
+
   // the previous row's threshold seeds the next search; it carries over from
   // strip to strip, since neighbouring strips are statistically alike
   uint32_t seed = 0u;
@@ -97,6 +90,19 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   const int logical = xcd_logical_id(hw, total);
   if (logical < 0) continue;
   __syncthreads();  // the previous strip's lists have been stored
+  // Everything derived from the lane id is derived again for every strip: kept
+  // across strips it would sit in spilled registers, and a reload from scratch
+  // costs more than the two or three instructions that recompute it.
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int half = lane >> 5;
+  const int wx = wave & 7;   // which 32 candidates of a tile
+  const int wy = wave >> 3;  // which half of the strip's rows
+  // a staged row, once in registers, lends its space to the candidate list
+  entry_t* cand = reinterpret_cast<entry_t*>(lds + wave * kStagePitch);
   const int split = logical / per_split;
   const int rem = logical - split * per_split;
   const int b = rem / a.ystrips;
