@@ -90,19 +90,6 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   const int logical = xcd_logical_id(hw, total);
   if (logical < 0) continue;
   __syncthreads();  // the previous strip's lists have been stored
-  // Everything derived from the lane id is derived again for every strip: kept
-  // across strips it would sit in spilled registers, and a reload from scratch
-  // costs more than the two or three instructions that recompute it.
-  int tid = threadIdx.x;
-  asm volatile("" : "+v"(tid));
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int l32 = lane & 31;
-  const int half = lane >> 5;
-  const int wx = wave & 7;   // which 32 candidates of a tile
-  const int wy = wave >> 3;  // which half of the strip's rows
-  // a staged row, once in registers, lends its space to the candidate list
-  entry_t* cand = reinterpret_cast<entry_t*>(lds + wave * kStagePitch);
   const int split = logical / per_split;
   const int rem = logical - split * per_split;
   const int b = rem / a.ystrips;
@@ -143,6 +130,21 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
         if (i < nt) core.slab(X, Y, lds, acc[i]);
     }
     __syncthreads();  // all fragment reads are done; the buffers become the staging area
+
+    // Everything derived from the lane id is derived here, after the product and
+    // again for every chunk: kept across the product (or across strips) it would
+    // only occupy, or spill, registers there, and a reload from scratch costs
+    // more than the two or three instructions that recompute it.
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+    const int wx = wave & 7;   // which 32 candidates of a tile
+    const int wy = wave >> 3;  // which half of the strip's rows
+    // a staged row, once in registers, lends its space to the candidate list
+    entry_t* cand = reinterpret_cast<entry_t*>(lds + wave * kStagePitch);
 
     // selection, sixteen rows of the strip per pass
     const int xc0 = xt0 * kTileX;
@@ -198,6 +200,11 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
     }
   }
 
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  uint32_t* sort_scratch = reinterpret_cast<uint32_t*>(lds + wave * kStagePitch);
   // each wave finishes the four rows it owns, two at a time
 #pragma unroll 1
   for (int g = 0; g < 4; g += 2) {
@@ -212,7 +219,7 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
         vals[rr] = y < Yext ? a.values + orow * a.k : nullptr;
         inds[rr] = y < Yext ? a.indices + orow * a.k : nullptr;
       }
-      sort_and_store_pair((lds_entry_ptr)list[ra], (lds_entry_ptr)list[rb], (lds_u32_ptr)cand,
+      sort_and_store_pair((lds_entry_ptr)list[ra], (lds_entry_ptr)list[rb], (lds_u32_ptr)sort_scratch,
                           vals[0], vals[1], inds[0], inds[1], a.k);
     } else {
 #pragma unroll
