@@ -28,8 +28,8 @@ PEAK_HBM_GBS = 8000.0
 # traffic = (2 * FETCH_SIZE + WRITE_SIZE) * 1024.  The counters cannot be read
 # from inside this process; the figures are those of the summaries in profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "min_bmm_large": (2 * 2.13965e6 + 2048) * 1024,      # profiles/min_kernel_min_bmm_large.txt
-    "topk_bmm": (2 * 785073 + 1.57286e6) * 1024,          # profiles/topk_kernel_topk_bmm.txt
+    "min_bmm_large": (2 * 2.03203e6 + 2048) * 1024,      # profiles/min_kernel_min_bmm_large.txt
+    "topk_bmm": (2 * 853429 + 1.71004e6) * 1024,          # profiles/topk_kernel_topk_bmm.txt
 }
 
 
