@@ -21,6 +21,8 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 PEAK_HBM_GBS = 8000.0
+PEAK_VALU_TOPS = 39.3           # 256 CUs x 64 lanes x 2.4 GHz: one fp32 vector instruction per lane and cycle
+                                # (packed fp32 is switched off in this build)
 
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc
 # (FETCH_SIZE, WRITE_SIZE: KiB per dispatch).  On this box FETCH_SIZE reads half
@@ -58,6 +60,19 @@ def make_workloads(torch, cmk, dev):
                        desc="min_bmm fp32 A[1,%d,%d] @ B[1,%d,%d], min+argmin over dim=-1" % (M, K, K, N),
                        cpu=cpu, cpu_rows=cpu_rows, rows=M, cpu_flop_per_row=2.0 * N * K,
                        cpu_expr="torch.bmm(A,B).min(-1)")
+
+    def min_dist_wl(name, distance, M, N, K):
+        # (a-b)^2 / |a-b| accumulation on the vector unit: two instructions per (m, n, k) either way
+        # (subtract + fused multiply-add for l2, subtract + add-of-absolute-value for l1)
+        op = cmk.MinBMMCUDA(distance=distance)
+
+        def make():
+            return randn(1, M, K, seed=0), randn(1, K, N, seed=1)
+
+        per = 3.0 if distance == "l2" else 2.0
+        W[name] = dict(make=make, run=lambda A, B: op(A, B, dim=-1), flop=per * M * N * K, valu_ops=2.0 * M * N * K,
+                       desc="min_bmm distance=%s fp32 A[1,%d,%d] vs B[1,%d,%d], min+argmin over dim=-1 "
+                            "(vector unit, %d flop per element pair and k)" % (distance, M, K, K, N, int(per)))
 
     def topk_wl(name, M, N, K, cpu_rows):
         op = cmk.TopkBMMCUDA()
@@ -117,6 +132,8 @@ def make_workloads(torch, cmk, dev):
     topk_wl("topk_bmm", 1048576, 1024, 256, cpu_rows=65536)
     bmm_wl("bmm", 128, 1024, 1024, 128)
     mbmm_wl("mbmm", 128, 1024, 1024, 64)
+    min_dist_wl("min_bmm_l2", "l2", 16384, 16384, 256)
+    min_dist_wl("min_bmm_l1", "l1", 16384, 16384, 256)
     return W
 
 
@@ -201,15 +218,24 @@ def main():
     args, ms, kern_ms = run_workload(torch, wl, a.steps, a.warmup)
     gflops = wl["flop"] / (ms * 1e-3) / 1e9
     achieved = wl["flop"] / (kern_ms * 1e-3) / 1e12
+    if "valu_ops" in wl:
+        ach = wl["valu_ops"] / (kern_ms * 1e-3) / 1e12
+        roof = {"bound": "valu", "achieved": round(ach, 2), "peak": PEAK_VALU_TOPS, "unit": "Tinstr/s (per lane)",
+                "frac": round(ach / PEAK_VALU_TOPS, 4), "traffic": None, "kernel_ms": round(kern_ms, 4)}
+        metric = "GFLOP/s of fused %s (flop as the workload states / time), fp32 vector unit" % a.workload
+    else:
+        roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload), "kernel_ms": round(kern_ms, 4)}
+        metric = ("GFLOP/s of fused %s (2*M*N*K / time), fp32 MFMA"
+                  % a.workload.split("_large")[0].split("_small")[0])
     out = {
-        "metric": "GFLOP/s of fused %s (2*M*N*K / time), fp32 MFMA" % a.workload.split("_large")[0].split("_small")[0],
+        "metric": metric,
         "value": round(gflops, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": wl["desc"], "name": a.workload},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload), "kernel_ms": round(kern_ms, 4)},
+        "roofline": roof,
     }
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, wl, args)
@@ -224,8 +250,11 @@ def main():
             steps = 5 if name == "topk_bmm" else 20
             args, ms_o, kern_o = run_workload(torch, w, steps, 3)
             rec = {"workload": w["desc"], "ms_per_step": round(ms_o, 4), "kernel_ms": round(kern_o, 4),
-                   "GFLOP/s": round(w["flop"] / (kern_o * 1e-3) / 1e9, 1),
-                   "frac_fp32_mfma_peak": round(w["flop"] / (kern_o * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
+                   "GFLOP/s": round(w["flop"] / (kern_o * 1e-3) / 1e9, 1)}
+            if "valu_ops" in w:
+                rec["frac_valu_issue_peak"] = round(w["valu_ops"] / (kern_o * 1e-3) / 1e12 / PEAK_VALU_TOPS, 4)
+            else:
+                rec["frac_fp32_mfma_peak"] = round(w["flop"] / (kern_o * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)
             if "bytes" in w:
                 rec["GB/s"] = round(w["bytes"] / (kern_o * 1e-3) / 1e9, 1)
                 rec["frac_hbm_peak"] = round(rec["GB/s"] / PEAK_HBM_GBS, 4)

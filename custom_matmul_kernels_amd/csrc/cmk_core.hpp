@@ -50,6 +50,10 @@ typedef const void __attribute__((address_space(1))) * global_void_ptr;
 typedef void __attribute__((address_space(3))) * lds_void_ptr;
 
 constexpr int kThreads = 256;
+// what one (x, y, k) triple contributes to an accumulator
+constexpr int kInner = 0;   // x*y, on the matrix pipe
+constexpr int kL2 = 1;      // (x-y)^2, vector unit
+constexpr int kL1 = 2;      // |x-y|,   vector unit
 constexpr int KC = 0;   // k-contiguous operand
 constexpr int RC = 1;   // row-contiguous operand
 
@@ -389,16 +393,98 @@ struct Core {
   }
 
   // acc += the current tile's product: S slabs of the flat sequence.
+  template <int DIST = kInner>
   __device__ __forceinline__ void tile(const Operand& X, const Operand& Y, float* lds,
                                        f32x16 (&acc)[BX][BY]) {
     static_assert(!Y_ONCE, "with Y_ONCE the kernel walks slabs itself: tiles inside k-slabs");
-    for (int s = 0; s < S; ++s) slab(X, Y, lds, acc);
+    for (int s = 0; s < S; ++s) slab<DIST>(X, Y, lds, acc);
+  }
+
+  // The distances other than the inner product have no matrix-pipe form.  They
+  // run on the vector unit over the same LDS slabs and into the same accumulator
+  // layout as the MFMA path (register r of a lane: X row acc_row(r, half) of the
+  // block, Y row lane % 32), so the kernels' epilogues do not change.  Per
+  // accumulator the k values are taken in ascending order with the reference's
+  // operations (kernels/bmm_helpers.cu:28-35, 46-52): d = x - y, then
+  // fmaf(d, d, c) or c + fabsf(d).  Zero-filled padding along k adds nothing.
+  template <int DIST>
+  __device__ __forceinline__ void dist_group(const float* xb, const float* yb, int kg,
+                                             f32x16 (&acc)[BX][BY]) {
+    const int l32 = tid & 31;
+    const int xw = ((tid >> 6) % WX) * BX * 32 + 4 * half;   // first X row of this half-wave
+    const int yl = ((tid >> 6) / WX) * BY * 32 + l32;        // this lane's first Y row
+    float y[BY][8];
+#pragma unroll
+    for (int by = 0; by < BY; ++by) {
+      if constexpr (YK == KC) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const f32x4 v = *reinterpret_cast<const f32x4*>(&yb[lds_pos<KC, TY, KS>(yl + 32 * by, kg * 8 + 4 * h)]);
+          y[by][4 * h] = v.x; y[by][4 * h + 1] = v.y; y[by][4 * h + 2] = v.z; y[by][4 * h + 3] = v.w;
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) y[by][k] = yb[(kg * 8 + k) * TY + yl + 32 * by];
+      }
+    }
+    auto add = [](float xv, float yv, float cv) {
+      const float d = xv - yv;
+      return DIST == kL2 ? __builtin_fmaf(d, d, cv) : cv + __builtin_fabsf(d);
+    };
+#pragma unroll
+    for (int bx = 0; bx < BX; ++bx)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const int row0 = xw + 32 * bx + 8 * rg;   // rows row0 .. row0+3 are registers 4rg .. 4rg+3
+        if constexpr (XK == KC) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float x[8];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              const f32x4 v = *reinterpret_cast<const f32x4*>(&xb[lds_pos<KC, TX, KS>(row0 + e, kg * 8 + 4 * h)]);
+              x[4 * h] = v.x; x[4 * h + 1] = v.y; x[4 * h + 2] = v.z; x[4 * h + 3] = v.w;
+            }
+#pragma unroll
+            for (int by = 0; by < BY; ++by)
+#pragma unroll
+              for (int k = 0; k < 8; ++k) acc[bx][by][4 * rg + e] = add(x[k], y[by][k], acc[bx][by][4 * rg + e]);
+          }
+        } else {
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(&xb[(kg * 8 + k) * TX + row0]);
+            const float x[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int by = 0; by < BY; ++by)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[bx][by][4 * rg + e] = add(x[e], y[by][k], acc[bx][by][4 * rg + e]);
+          }
+        }
+      }
   }
 
   // acc += one slab of the flat sequence.
+  template <int DIST = kInner>
   __device__ __forceinline__ void slab(const Operand& X, const Operand& Y, float* lds,
                                        f32x16 (&acc)[BX][BY]) {
-    {
+    if constexpr (DIST != kInner) {
+      float* cur = xbuf(lds, it);
+      const float* ycur = ybuf(lds, it, cs);
+      const bool has1 = it + 1 < iters;
+      const bool has2 = it + 2 < iters;
+      issue_y(Y);
+#pragma unroll 1   // a k-group is 2 * 64 * BX * BY * 8 vector instructions: keep the code in the instruction cache
+      for (int kg = 0; kg < NG; ++kg) dist_group<DIST>(cur, ycur, kg, acc);
+      if (has1) {
+        wait_loads();     // this wave's part of slab it+1 is in LDS
+        __syncthreads();  // everyone's is, and nobody reads `cur` any more
+        pend_xbuf = has2 ? cur : nullptr;
+        issue_pending_x(X);
+      }
+      ++it;
+      if (Y_ONCE && ++ct == nt) { ct = 0; ++cs; }
+    } else {
       float* cur = xbuf(lds, it);
       const float* nxt = xbuf(lds, it + 1);
       const int ns = (Y_ONCE && ct + 1 == nt) ? cs + 1 : cs;   // k-slab of the next flat slab

@@ -32,7 +32,7 @@ struct MinArgs {
   int total;                    // work-groups with real work slots (before XCD padding)
 };
 
-template <int XK, int YK>
+template <int XK, int YK, int DIST>
 __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
   using C = Core<XK, YK, 2, 2, 2, 2, 32, kReadsPaired, true>;
   __shared__ __attribute__((aligned(16))) float lds[C::ldsFloats];
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    core.tile(X, Y, lds, acc);
+    core.template tile<DIST>(X, Y, lds, acc);
     // fold this tile into the running minimum; indices ascend within a lane,
     // so a strict '<' keeps the first occurrence
     const int xb = xt * C::TX + wx * 64;
@@ -205,8 +205,6 @@ extern "C" int cmk_min_bmm_f32(const float* A, const float* B, float* values, lo
   if (dim != 1 && dim != 2) return fail(CMK_ERR_INVALID_ARG, "cmk_min_bmm_f32: dim must be 1 or 2");
   if (distance < CMK_DIST_INNER || distance > CMK_DIST_L1)
     return fail(CMK_ERR_INVALID_ARG, "cmk_min_bmm_f32: unknown distance %d", distance);
-  if (distance != CMK_DIST_INNER)
-    return fail(CMK_ERR_UNSUPPORTED, "cmk_min_bmm_f32: only distance \"inner\" is implemented");
   const int Xext = dim == 2 ? d->N : d->M;
   const int Yext = dim == 2 ? d->M : d->N;
   if (Xext == 0) return fail(CMK_ERR_INVALID_ARG, "cmk_min_bmm_f32: reduction over an empty axis");
@@ -243,10 +241,18 @@ extern "C" int cmk_min_bmm_f32(const float* A, const float* B, float* values, lo
   a.total = (int)total;
   const dim3 grid((unsigned)(((total + 7) / 8) * 8)), block(kThreads);
   hipStream_t st = (hipStream_t)stream;
-  if (xk == KC && yk == KC) hipLaunchKernelGGL((min_kernel<KC, KC>), grid, block, 0, st, a);
-  else if (xk == KC && yk == RC) hipLaunchKernelGGL((min_kernel<KC, RC>), grid, block, 0, st, a);
-  else if (xk == RC && yk == KC) hipLaunchKernelGGL((min_kernel<RC, KC>), grid, block, 0, st, a);
-  else hipLaunchKernelGGL((min_kernel<RC, RC>), grid, block, 0, st, a);
+#define CMK_MIN_LAUNCH(DIST)                                                                        \
+  do {                                                                                           \
+    if (xk == KC && yk == KC) hipLaunchKernelGGL((min_kernel<KC, KC, DIST>), grid, block, 0, st, a);      \
+    else if (xk == KC && yk == RC) hipLaunchKernelGGL((min_kernel<KC, RC, DIST>), grid, block, 0, st, a); \
+    else if (xk == RC && yk == KC) hipLaunchKernelGGL((min_kernel<RC, KC, DIST>), grid, block, 0, st, a); \
+    else hipLaunchKernelGGL((min_kernel<RC, RC, DIST>), grid, block, 0, st, a);                           \
+  } while (0)
+  static_assert(CMK_DIST_INNER == kInner && CMK_DIST_L2 == kL2 && CMK_DIST_L1 == kL1, "distance codes");
+  if (distance == CMK_DIST_INNER) CMK_MIN_LAUNCH(kInner);
+  else if (distance == CMK_DIST_L2) CMK_MIN_LAUNCH(kL2);
+  else CMK_MIN_LAUNCH(kL1);
+#undef CMK_MIN_LAUNCH
   if (int e = hip_status(hipGetLastError(), "cmk_min_bmm_f32 launch")) return e;
   if (a.splits > 1) {
     const long long rows = (long long)d->L * Yext;

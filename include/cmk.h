@@ -46,7 +46,11 @@ extern "C" {
 #define CMK_OP_TOPK_BMM 3
 #define CMK_OP_TOPK_1D  4
 
-/* accumulate functions (reference kernels/bmm_helpers.cu:20-60) */
+/* accumulate functions of min_bmm / topk_bmm (reference kernels/bmm_helpers.cu:20-60;
+ * selected by the `distance` constructor argument, minbmm.py:12-19, topkbmm.py:15-22).
+ * INNER runs on the matrix pipe; L2 and L1 have no matrix form and run on the
+ * vector unit, in the reference's order of operations (d = a - b, then
+ * fmaf(d, d, c) or c + fabsf(d), k ascending), a few times slower. */
 #define CMK_DIST_INNER 0   /* c += a*b        ("madd")       */
 #define CMK_DIST_L2    1   /* c += (a-b)^2    ("squared_l2") */
 #define CMK_DIST_L1    2   /* c += |a-b|      ("l1")         */
@@ -84,8 +88,9 @@ int cmk_mbmm_f32(const float* A, const float* B, float* C,
                  const cmk_gemm_desc* d, void* stream);
 
 /*
- * Fused min/argmin of C = A@B along `dim` of C[L][M][N] (1 = over m, output
- * [L][N]; 2 = over n, output [L][M]) without storing C.  `values` is fp32,
+ * Fused min/argmin of C = A@B (or of the accumulated distance CMK_DIST_*
+ * between the rows of A and the columns of B) along `dim` of C[L][M][N] (1 =
+ * over m, output [L][N]; 2 = over n, output [L][M]) without storing C.  `values` is fp32,
  * `indices` int64; every output element is written; exact ties resolve to
  * the lowest index.  Replaces the launch of min_bmm_{nn,nt,tn,tt}
  * (reference minbmm.py:132-143, kernels/minbmm.cu:347-440).
@@ -96,8 +101,9 @@ int cmk_min_bmm_f32(const float* A, const float* B,
                     void* workspace, size_t workspace_bytes, void* stream);
 
 /*
- * Fused top-k (largest, sorted descending, 0 < k <= 128) of C = A@B along
- * `dim` of C[L][M][N]: dim == 2 gives [L][M][k], dim == 1 gives [L][N][k].
+ * Fused top-k (largest, sorted descending, 0 < k <= 128) of C = A@B (or of
+ * the accumulated distance CMK_DIST_*; still the largest k) along `dim` of
+ * C[L][M][N]: dim == 2 gives [L][M][k], dim == 1 gives [L][N][k].
  * `values` fp32 and `indices` int64 are dense with row pitch k.  When fewer
  * than k candidates exist the trailing slots hold -inf / -1.  Replaces the
  * launch of topk_bmm_{nn,nt,tn,tt}

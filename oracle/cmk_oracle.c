@@ -11,7 +11,10 @@
  *
  * Pinned by tests/test_oracle.py: exact-integer fixtures computed with int64
  * arithmetic, float64 closed forms, brute-force loops on tiny shapes, and the
- * 0/1 principle for the sorting network.
+ * 0/1 principle for the sorting network.  The (a-b)^2 and |a-b| accumulate
+ * functions (:28-35, :46-52) are run by none of the reference's notebooks; they
+ * are pinned by exact int64 distances, a brute-force loop in the reference's
+ * order of operations, torch.cdist in float64 and the zero-distance case.
  */
 #include <math.h>
 #include <stdint.h>

@@ -97,6 +97,63 @@ def test_c_layer_agrees_with_torch_layer_on_floats():
         assert O.check_topk(torch.from_numpy(v), torch.from_numpy(i), A, B, 128, dim) <= 8
 
 
+@pytest.mark.parametrize("code,p", [(1, 2), (2, 1)])
+def test_distances_against_closed_forms(code, p):
+    """(a-b)^2 and |a-b| accumulation (reference kernels/bmm_helpers.cu:28-35,
+    46-52).  The reference's notebooks never run these, so they are pinned by
+    what the mathematics fixes: integer inputs computed exactly in int64, a
+    brute-force loop in the reference's order of operations, torch.cdist in
+    float64, and special cases (identical vectors, a single k)."""
+    rng = np.random.default_rng(5)
+    # exact: small integers, every partial sum is an integer below 2^24
+    Ai = rng.integers(-9, 10, size=(2, 17, 13))
+    Bi = rng.integers(-9, 10, size=(2, 13, 21))
+    diff = Ai[:, :, :, None] - Bi[:, None, :, :]                     # [l, m, k, n]
+    D = (diff ** 2 if p == 2 else np.abs(diff)).sum(2)               # int64 [l, m, n]
+    for dim in (1, 2):
+        v, i = O.c_min_bmm(Ai.astype(np.float32), Bi.astype(np.float32), dim, code)
+        assert np.array_equal(v, D.min(dim).astype(np.float32))
+        assert np.array_equal(i, D.argmin(dim))                      # first minimum = lowest index
+        tv, ti = O.c_topk_bmm(Ai.astype(np.float32), Bi.astype(np.float32), 128, dim, code)
+        red = D.shape[dim]
+        want = -np.sort(-D, axis=dim).swapaxes(dim, 2)[..., :red]    # largest first
+        assert np.array_equal(tv[..., :red], want.astype(np.float32))
+        assert np.isneginf(tv[..., red:]).all()
+        picked = np.take_along_axis(D.swapaxes(dim, 2), ti[..., :red], axis=2)
+        assert np.array_equal(picked, want)                          # indices point at their values
+    # brute force in the reference's order: one accumulator, k ascending
+    A, B = seeded(1, 6, 5, 11, seed=9)
+    v, i = O.c_min_bmm(A.numpy(), B.numpy(), 2, code)
+    for m in range(6):
+        best = None
+        for n in range(5):
+            acc = np.float32(0)
+            for k in range(11):
+                d = np.float32(A[0, m, k].item()) - np.float32(B[0, k, n].item())
+                if p == 2:   # fmaf(d, d, acc): one rounding
+                    acc = np.float32(np.float64(d) * np.float64(d) + np.float64(acc))
+                else:
+                    acc = np.float32(acc + np.abs(d))
+            if best is None or acc < best[0]:
+                best = (acc, n)
+        assert v[0, m] == best[0] and i[0, m] == best[1]
+    # float64 closed form on random floats
+    A, B = seeded(2, 40, 50, 33, seed=10)
+    cd = torch.cdist(A.double(), B.double().transpose(1, 2), p=p)
+    cd = cd ** 2 if p == 2 else cd
+    for dim in (1, 2):
+        v, i = O.c_min_bmm(A.numpy(), B.numpy(), dim, code)
+        assert np.allclose(v, cd.min(dim)[0].numpy(), rtol=1e-5, atol=1e-4)
+        tv, ti = O.c_topk_bmm(A.numpy(), B.numpy(), 128, dim, code)
+        red = cd.shape[dim]
+        assert np.allclose(tv[..., :red], cd.topk(red, dim)[0].transpose(dim, 2).numpy()[..., :red], rtol=1e-5, atol=1e-4)
+    # identical vectors are at distance exactly 0 and win the minimum
+    A = torch.randn(1, 4, 7)
+    B = A[0].t().contiguous()[None]                                  # column j of B = row j of A
+    v, i = O.c_min_bmm(A.numpy(), B.numpy(), 2, code)
+    assert (v == 0).all() and np.array_equal(i[0], np.arange(4))
+
+
 def test_mask_precedence():
     """block mask beats thread mask beats element mask; the element mask byte
     multiplies (reference kernels/mbmm.cu:127-128, 251-255, 360-363)."""

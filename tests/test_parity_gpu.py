@@ -191,6 +191,61 @@ def test_min_bmm_integer_cases_and_ties(device, name, dim):
         assert torch.equal(i.cpu(), torch.from_numpy(g["%s_min%d_idx" % (name, dim)].astype(np.int64)))
 
 
+DIST_SHAPES = [(1, 5, 7, 3), (2, 130, 140, 33), (1, 300, 260, 64), (1, 64, 1100, 40)]
+
+
+@pytest.mark.parametrize("distance", ["l2", "l1"])
+@pytest.mark.parametrize("dim", [1, 2])
+@pytest.mark.parametrize("mode", ["nn", "tt", "nt"])
+@pytest.mark.parametrize("shape", DIST_SHAPES)
+def test_min_bmm_distances_match_oracle(device, shape, mode, dim, distance):
+    """(a-b)^2 and |a-b| accumulate on the vector unit in the reference's order
+    of operations: values are bit-equal to the C oracle, ties go to the lowest
+    index."""
+    say("min", distance, shape, mode, dim)
+    L, M, N, K = shape
+    A, B = seeded(L, M, N, K, seed=12)
+    Ad, Bd = place(A, B, mode, device)
+    v, i = MinBMMCUDA(distance=distance)(Ad, Bd, dim=dim)
+    code = {"l2": 1, "l1": 2}[distance]
+    cv, ci = O.c_min_bmm(A.numpy(), B.numpy(), dim, code)
+    assert torch.equal(v.cpu(), torch.from_numpy(cv))
+    assert torch.equal(i.cpu(), torch.from_numpy(ci).long())
+    # closed form: torch.cdist between the rows of A and the columns of B
+    p = 2 if distance == "l2" else 1
+    D = torch.cdist(A.double(), B.double().transpose(1, 2), p=p)
+    if p == 2:
+        D = D ** 2
+    want = D.min(dim)[0]
+    assert torch.allclose(v.cpu().double(), want, rtol=1e-4, atol=1e-3 * K ** 0.5)
+
+
+@pytest.mark.parametrize("distance", ["euclidean", "manhattan"])
+@pytest.mark.parametrize("dim", [1, 2])
+@pytest.mark.parametrize("shape", [(1, 5, 7, 3), (2, 130, 300, 33), (1, 70, 2500, 16)])
+def test_topk_bmm_distances_match_oracle(device, shape, dim, distance):
+    """Largest k of the accumulated distances, as the reference's kernels would
+    select them (its top-k always keeps the largest values)."""
+    say("topk", distance, shape, dim)
+    L, M, N, K = shape
+    A, B = seeded(L, M, N, K, seed=13)
+    v, i = TopkBMMCUDA(distance=distance)(A.to(device), B.to(device), k=128, dim=dim)
+    code = {"euclidean": 1, "manhattan": 2}[distance]
+    cv, ci = O.c_topk_bmm(A.numpy(), B.numpy(), 128, dim, code)
+    red = M if dim == 1 else N
+    kk = min(128, red)
+    assert torch.equal(v.cpu()[..., :kk], torch.from_numpy(cv)[..., :kk])
+    # indices: equal wherever the value is not repeated in the row
+    gv = v.cpu()[..., :kk]
+    uniq = torch.ones_like(gv, dtype=torch.bool)
+    uniq[..., 1:] &= gv[..., 1:] != gv[..., :-1]
+    uniq[..., :-1] &= gv[..., :-1] != gv[..., 1:]
+    uniq &= gv != gv[..., -1:]          # a tie with the first value left out may pick either
+    gi, wi = i.cpu()[..., :kk], torch.from_numpy(ci).long()[..., :kk]
+    bad = (gi != wi) & uniq
+    assert not bad.any(), (bad.nonzero()[:5], gi[bad][:5], wi[bad][:5], gv[bad][:5])
+
+
 def test_min_bmm_dims_2d_negative_and_determinism(device):
     A, B = seeded(1, 300, 500, 48, seed=8)
     op = MinBMMCUDA()
