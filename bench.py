@@ -32,6 +32,7 @@ PEAK_VALU_TOPS = 39.3           # 256 CUs x 64 lanes x 2.4 GHz: one fp32 vector 
 MEASURED_TRAFFIC_BYTES = {
     "min_bmm_large": (2 * 2.03203e6 + 2048) * 1024,      # profiles/min_kernel_min_bmm_large.txt
     "topk_bmm": (2 * 853429 + 1.71004e6) * 1024,          # profiles/topk_kernel_topk_bmm.txt
+    "derive_masks_4GiB": (2 * 2.09726e6 + 66696.9) * 1024,  # profiles/derive_masks_kernel_4GiB.txt
 }
 
 
@@ -107,14 +108,26 @@ def make_workloads(torch, cmk, dev):
             tiles = torch.rand(L, M // 128, N // 128, generator=g) < 0.5
             keep = tiles.repeat_interleave(128, 1).repeat_interleave(128, 2)
             fm = torch.tril(torch.ones(M, N)).bool()[None] & keep
-            bm, tm, em = cmk.derive_masks(fm)
+            bm, tm, em = cmk.derive_masks(fm.to(dev))
             kept_tiles = int(bm.sum())
-            return A, B, bm.to(dev), tm.to(dev), em.to(dev), kept_tiles
+            return A, B, bm, tm, em, kept_tiles
 
         W[name] = dict(make=make, run=lambda A, B, bm, tm, em, kt: op(A, B, bm, tm, em),
                        flop=2.0 * L * M * N * K,
                        desc="mbmm fp32 A[%d,%d,%d] @ B[%d,%d,%d], tril & tile-Bernoulli(0.5) mask" % (L, M, K, L, K, N),
                        bytes=4.0 * L * (M * N + M * K + K * N) + L * M * N + L * (M // 8) * (N // 8))
+
+    def masks_wl(name, L, M, N):
+        # byte work: reads the element mask once, writes 1/64 + 1/16384 of it
+        def make():
+            g = torch.Generator().manual_seed(1)
+            tiles = (torch.rand(L, M // 128, N // 128, generator=g) < 0.5).to(dev)
+            keep = tiles.repeat_interleave(128, 1).repeat_interleave(128, 2)
+            return (torch.tril(torch.ones(M, N, device=dev)).bool()[None] & keep,)
+
+        W[name] = dict(make=make, run=lambda fm: cmk.derive_masks(fm), flop=0.0, dtype="u8",
+                       desc="derive_masks of a bool mask [%d,%d,%d] (block + thread masks)" % (L, M, N),
+                       bytes=1.0 * L * M * N + L * (M // 8) * (N // 8) + L * (M // 128) * (N // 128))
 
     def copy_wl(name, nbytes):
         # a plain device copy of known size: the yardstick the HBM counters are scaled by
@@ -132,6 +145,8 @@ def make_workloads(torch, cmk, dev):
     topk_wl("topk_bmm", 1048576, 1024, 256, cpu_rows=65536)
     bmm_wl("bmm", 128, 1024, 1024, 128)
     mbmm_wl("mbmm", 128, 1024, 1024, 64)
+    masks_wl("derive_masks", 128, 1024, 1024)
+    masks_wl("derive_masks_4GiB", 1024, 2048, 2048)
     min_dist_wl("min_bmm_l2", "l2", 16384, 16384, 256)
     min_dist_wl("min_bmm_l1", "l1", 16384, 16384, 256)
     return W
@@ -218,7 +233,13 @@ def main():
     args, ms, kern_ms = run_workload(torch, wl, a.steps, a.warmup)
     gflops = wl["flop"] / (ms * 1e-3) / 1e9
     achieved = wl["flop"] / (kern_ms * 1e-3) / 1e12
-    if "valu_ops" in wl:
+    if wl["flop"] == 0:
+        ach = wl["bytes"] / (kern_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
+                "kernel_ms": round(kern_ms, 4)}
+        metric = "GB/s of %s (algorithmic bytes / time)" % a.workload
+    elif "valu_ops" in wl:
         ach = wl["valu_ops"] / (kern_ms * 1e-3) / 1e12
         roof = {"bound": "valu", "achieved": round(ach, 2), "peak": PEAK_VALU_TOPS, "unit": "Tinstr/s (per lane)",
                 "frac": round(ach / PEAK_VALU_TOPS, 4), "traffic": None, "kernel_ms": round(kern_ms, 4)}
@@ -231,9 +252,10 @@ def main():
                   % a.workload.split("_large")[0].split("_small")[0])
     out = {
         "metric": metric,
-        "value": round(gflops, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "value": round(gflops, 1) if wl["flop"] > 0 else round(wl["bytes"] / (ms * 1e-3) / 1e9, 1),
+        "unit": "GFLOP/s" if wl["flop"] > 0 else "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": wl.get("dtype", "f32"), "data": "synthetic",
         "config": {"workload": wl["desc"], "name": a.workload},
         "roofline": roof,
     }
@@ -249,9 +271,12 @@ def main():
                 continue
             steps = 5 if name == "topk_bmm" else 20
             args, ms_o, kern_o = run_workload(torch, w, steps, 3)
-            rec = {"workload": w["desc"], "ms_per_step": round(ms_o, 4), "kernel_ms": round(kern_o, 4),
-                   "GFLOP/s": round(w["flop"] / (kern_o * 1e-3) / 1e9, 1)}
-            if "valu_ops" in w:
+            rec = {"workload": w["desc"], "ms_per_step": round(ms_o, 4), "kernel_ms": round(kern_o, 4)}
+            if w["flop"] > 0:
+                rec["GFLOP/s"] = round(w["flop"] / (kern_o * 1e-3) / 1e9, 1)
+            if w["flop"] == 0:
+                pass
+            elif "valu_ops" in w:
                 rec["frac_valu_issue_peak"] = round(w["valu_ops"] / (kern_o * 1e-3) / 1e12 / PEAK_VALU_TOPS, 4)
             else:
                 rec["frac_fp32_mfma_peak"] = round(w["flop"] / (kern_o * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)

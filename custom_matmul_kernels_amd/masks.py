@@ -1,32 +1,44 @@
-"""Derivation of the three mask levels MBMMCUDA takes from one boolean mask,
-following colab/test_mbmm.ipynb:1295-1313 of the reference: the element mask is
-the mask itself, the thread mask counts kept elements per 8x8 micro-tile
-(0..64) and the block mask flags 128x128 tiles with any kept element.  Extents
-that are not multiples of 8 / 128 are padded with zeros (the notebook only
-handles multiples)."""
+"""The three mask levels MBMMCUDA takes, derived on the GPU from one boolean
+mask by libcmk's ``cmk_derive_masks_u8``: the element mask is the mask itself,
+the thread mask counts kept elements per 8x8 micro-tile (0..64) and the block
+mask flags 128x128 tiles with any kept element -- the rule callers of the
+reference apply with tensor reductions (reference
+colab/test_mbmm.ipynb:1295-1313).  Extents that are not multiples of 8 / 128
+are padded with zeros (the notebook only handles multiples)."""
 import math
 
 import torch
-import torch.nn.functional as F
+
+from . import _lib
 
 
 def derive_masks(final_mask):
-    """final_mask: bool [m, n] or [l, m, n] -> (block_mask, thread_mask,
-    element_mask), all uint8, in the argument order of MBMMCUDA.__call__."""
-    fm = final_mask.bool()
-    squeeze = fm.dim() == 2
+    """final_mask: bool or uint8 device tensor [m, n] or [l, m, n] ->
+    (block_mask, thread_mask, element_mask), all uint8 on the same device, in
+    the argument order of MBMMCUDA.__call__.  A bool mask is reinterpreted, not
+    copied; a uint8 mask is used as given (any non-zero byte counts as kept,
+    and the product is multiplied by the byte, as reference
+    kernels/mbmm.cu:127-128 does)."""
+    if final_mask.dtype not in (torch.bool, torch.uint8):
+        raise TypeError("the mask must be torch.bool or torch.uint8, got %s" % final_mask.dtype)
+    if final_mask.dim() not in (2, 3):
+        raise ValueError("the mask needs to be 2d or 3d")
+    if final_mask.device.type != "cuda":
+        raise ValueError("the mask must be a device tensor (got device %s)" % final_mask.device)
+    lib = _lib.load()
+    em = final_mask.contiguous()
+    if em.dtype == torch.bool:
+        em = em.view(torch.uint8)
+    squeeze = em.dim() == 2
+    e3 = em[None] if squeeze else em
+    l, m, n = e3.shape
+    dev = em.device
+    block_mask = torch.empty((l, math.ceil(m / 128), math.ceil(n / 128)), dtype=torch.uint8, device=dev)
+    thread_mask = torch.empty((l, math.ceil(m / 8), math.ceil(n / 8)), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        _lib.check(lib.cmk_derive_masks_u8(e3.data_ptr(), block_mask.data_ptr(), thread_mask.data_ptr(),
+                                           l, m, n, stream))
     if squeeze:
-        fm = fm[None]
-    l, m, n = fm.shape
-    m8, n8 = math.ceil(m / 8), math.ceil(n / 8)
-    m128, n128 = math.ceil(m / 128), math.ceil(n / 128)
-    u = fm.to(torch.uint8)
-    p8 = F.pad(u, (0, n8 * 8 - n, 0, m8 * 8 - m))
-    thread_mask = p8.view(l, m8, 8, n8, 8).sum(dim=(2, 4), dtype=torch.int32).to(torch.uint8)
-    p128 = F.pad(u, (0, n128 * 128 - n, 0, m128 * 128 - m))
-    block_mask = (p128.view(l, m128, 128, n128, 128).sum(dim=(2, 4), dtype=torch.int32) > 0)
-    block_mask = block_mask.to(torch.uint8)
-    element_mask = u.contiguous()
-    if squeeze:
-        return block_mask[0], thread_mask[0], element_mask[0]
-    return block_mask, thread_mask, element_mask
+        return block_mask[0], thread_mask[0], em
+    return block_mask, thread_mask, em

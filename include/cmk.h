@@ -88,6 +88,18 @@ int cmk_mbmm_f32(const float* A, const float* B, float* C,
                  const cmk_gemm_desc* d, void* stream);
 
 /*
+ * Derives mbmm's coarse masks from an element mask [Lm][M][N] (uint8, any
+ * non-zero byte = kept; a torch.bool tensor's storage qualifies):
+ * thread_mask[Lm][ceil(M/8)][ceil(N/8)] = kept elements per 8x8 micro-tile
+ * (0..64), block_mask[Lm][ceil(M/128)][ceil(N/128)] = 1 where the 128x128 tile
+ * keeps any.  Elements beyond M or N count as dropped.  The reference has no
+ * kernel for this: its callers derive the masks with tensor reductions
+ * (reference colab/test_mbmm.ipynb:1295-1313), which this entry point replaces.
+ */
+int cmk_derive_masks_u8(const uint8_t* element_mask, uint8_t* block_mask,
+                        uint8_t* thread_mask, int Lm, int M, int N, void* stream);
+
+/*
  * Fused min/argmin of C = A@B (or of the accumulated distance CMK_DIST_*
  * between the rows of A and the columns of B) along `dim` of C[L][M][N] (1 =
  * over m, output [L][N]; 2 = over n, output [L][M]) without storing C.  `values` is fp32,

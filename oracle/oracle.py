@@ -135,6 +135,30 @@ def ref_bmm(A, B):
     return torch.bmm(A, B)
 
 
+def ref_derive_masks(final_mask):
+    """(block_mask, thread_mask, element_mask), uint8, from a bool mask [m, n] or
+    [l, m, n]: counts per 8x8 micro-tile and any-kept flags per 128x128 tile, as
+    reference colab/test_mbmm.ipynb:1295-1313 forms them, with zero padding for
+    extents that are not multiples of 8 / 128."""
+    fm = final_mask != 0
+    squeeze = fm.dim() == 2
+    if squeeze:
+        fm = fm[None]
+    l, m, n = fm.shape
+    m8, n8 = math.ceil(m / 8), math.ceil(n / 8)
+    m128, n128 = math.ceil(m / 128), math.ceil(n / 128)
+    u = fm.to(torch.uint8)
+    pad = torch.nn.functional.pad
+    p8 = pad(u, (0, n8 * 8 - n, 0, m8 * 8 - m))
+    thread_mask = p8.view(l, m8, 8, n8, 8).sum(dim=(2, 4), dtype=torch.int32).to(torch.uint8)
+    p128 = pad(u, (0, n128 * 128 - n, 0, m128 * 128 - m))
+    block_mask = (p128.view(l, m128, 128, n128, 128).sum(dim=(2, 4), dtype=torch.int32) > 0).to(torch.uint8)
+    element_mask = (final_mask.to(torch.uint8) if final_mask.dtype == torch.bool else final_mask).contiguous()
+    if squeeze:
+        return block_mask[0], thread_mask[0], element_mask
+    return block_mask, thread_mask, element_mask
+
+
 def ref_mbmm(A, B, final_mask):
     """final_mask: bool, True = keep (colab/test_mbmm.ipynb:1342-1343)."""
     C = torch.bmm(A, B)

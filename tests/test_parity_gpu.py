@@ -102,8 +102,10 @@ def test_mbmm_matches_oracle(device, shape, share):
     L, M, N, K = shape
     A, B = seeded(L, M, N, K, seed=6)
     fm = random_masks(L, M, N, seed=7, share=share)
-    bm, tm, em = derive_masks(fm)
-    C = MBMMCUDA(share_mask=share)(A.to(device), B.to(device), bm.to(device), tm.to(device), em.to(device))
+    bm, tm, em = O.ref_derive_masks(fm)
+    dbm, dtm, dem = derive_masks(fm.to(device))
+    assert torch.equal(dbm.cpu(), bm) and torch.equal(dtm.cpu(), tm) and torch.equal(dem.cpu(), em)
+    C = MBMMCUDA(share_mask=share)(A.to(device), B.to(device), dbm, dtm, dem)
     full = fm[None].expand(L, -1, -1) if share else fm
     want = O.ref_mbmm(A, B, full)
     O.check_values(C.cpu(), want, K, "mbmm")
@@ -113,12 +115,63 @@ def test_mbmm_matches_oracle(device, shape, share):
             O.c_mbmm(A.numpy(), B.numpy(), bm.numpy(), tm.numpy(), em.numpy(), share)), K, "mbmm vs C")
 
 
+MASK_SHAPES = [(1, 1, 1), (2, 130, 140), (1, 128, 128), (3, 256, 384), (2, 77, 9), (1, 1000, 1040),
+               (2, 136, 272), (1, 8, 2049)]
+
+
+@pytest.mark.parametrize("kind", ["bernoulli", "tril", "sparse", "bytes"])
+@pytest.mark.parametrize("shape", MASK_SHAPES)
+def test_derive_masks_matches_oracle(device, shape, kind):
+    """Bit-exact against the oracle's derivation: aligned and unaligned row
+    pitches, ragged extents, 2-D (shared) masks, a storage offset that breaks
+    16-byte alignment, and uint8 masks whose kept bytes are not 1."""
+    say("derive_masks", shape, kind)
+    L, M, N = shape
+    g = torch.Generator().manual_seed(11)
+    if kind == "bernoulli":
+        fm = torch.rand(L, M, N, generator=g) < 0.5
+    elif kind == "tril":
+        fm = torch.tril(torch.ones(M, N)).bool()[None].expand(L, -1, -1).contiguous()
+    elif kind == "sparse":
+        fm = torch.rand(L, M, N, generator=g) < 0.0005
+    else:
+        fm = (torch.randint(0, 256, (L, M, N), generator=g, dtype=torch.int32)
+              * (torch.rand(L, M, N, generator=g) < 0.3)).to(torch.uint8)
+    for mask in (fm, fm[0]):
+        bm, tm, em = O.ref_derive_masks(mask)
+        dbm, dtm, dem = derive_masks(mask.to(device))
+        assert dbm.dtype == dtm.dtype == dem.dtype == torch.uint8
+        assert torch.equal(dbm.cpu(), bm) and torch.equal(dtm.cpu(), tm) and torch.equal(dem.cpu(), em)
+    # the same mask at an odd byte offset inside a larger allocation
+    flat = torch.zeros(fm.numel() + 3, dtype=fm.dtype, device=device)
+    flat[3:] = fm.to(device).reshape(-1)
+    bm, tm, em = O.ref_derive_masks(fm)
+    dbm, dtm, dem = derive_masks(flat[3:].view(L, M, N))
+    assert torch.equal(dbm.cpu(), bm) and torch.equal(dtm.cpu(), tm) and torch.equal(dem.cpu(), em)
+
+
+def test_derive_masks_full_size_properties(device):
+    """At the mbmm benchmark's size: counts add up to the number of kept
+    elements, a block is flagged exactly when one of its counts is non-zero,
+    and the result equals the oracle's."""
+    L, M, N = 128, 1024, 1024
+    g = torch.Generator().manual_seed(5)
+    keep = torch.rand(L, M // 128, N // 128, generator=g) < 0.5
+    fm = torch.tril(torch.ones(M, N)).bool()[None] & keep.repeat_interleave(128, 1).repeat_interleave(128, 2)
+    dbm, dtm, dem = derive_masks(fm.to(device))
+    assert int(dtm.sum(dtype=torch.int64)) == int(fm.sum())
+    per_block = dtm.view(L, M // 128, 16, N // 128, 16).sum(dim=(2, 4), dtype=torch.int32)
+    assert torch.equal(per_block > 0, dbm.bool())
+    bm, tm, em = O.ref_derive_masks(fm)
+    assert torch.equal(dbm.cpu(), bm) and torch.equal(dtm.cpu(), tm)
+
+
 def test_mbmm_mask_precedence_and_integer_exactness(device):
     g = golden()
     for name in INT_CASES:
         A, B = golden_inputs(g, name)
-        bm, tm, em = derive_masks(torch.from_numpy(g[name + "_mask"]))
-        C = MBMMCUDA(share_mask=True)(A.to(device), B.to(device), bm.to(device), tm.to(device), em.to(device))
+        bm, tm, em = derive_masks(torch.from_numpy(g[name + "_mask"]).to(device))
+        C = MBMMCUDA(share_mask=True)(A.to(device), B.to(device), bm, tm, em)
         assert torch.equal(C.cpu(), torch.from_numpy(g[name + "_Cmasked"].astype(np.float32)))
     # inconsistent masks: block beats thread beats element, the byte multiplies
     A, B = seeded(1, 130, 140, 8, seed=7)

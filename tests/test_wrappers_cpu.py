@@ -6,6 +6,7 @@ import torch
 
 from custom_matmul_kernels_amd import (BMMCUDA, MBMMCUDA, MinBMMCUDA, TopkBMMCUDA, _common,
                                        derive_masks)
+from oracle import oracle as O
 
 
 def test_mode_from_strides():
@@ -90,10 +91,19 @@ def test_shape_and_dtype_checks_fire_before_any_launch():
            torch.zeros(1, 1, 1, dtype=u8), torch.zeros(1, 8, 8, dtype=u8), mode="tn")
 
 
-def test_derive_masks_follows_the_notebook_rule():
+def test_derive_masks_rejects_host_tensors_and_other_dtypes():
+    with pytest.raises(ValueError):
+        derive_masks(torch.ones(8, 8, dtype=torch.bool))
+    with pytest.raises(TypeError):
+        derive_masks(torch.ones(8, 8))
+    with pytest.raises(ValueError):
+        derive_masks(torch.ones(8, dtype=torch.bool))
+
+
+def test_oracle_mask_derivation_follows_the_notebook_rule():
     m, n = 256, 384
     fm = torch.tril(torch.ones(m, n)).bool()
-    bm, tm, em = derive_masks(fm)
+    bm, tm, em = O.ref_derive_masks(fm)
     # colab/test_mbmm.ipynb:1303-1313 for shapes that are multiples of 8 / 128
     want_tm = fm.view(m // 8, 8, n // 8, 8).sum(dim=1).sum(dim=-1).to(torch.uint8)
     want_bm = fm.view(m // 128, 128, n // 128, 128).sum(dim=1).sum(dim=-1).bool().to(torch.uint8)
@@ -102,9 +112,17 @@ def test_derive_masks_follows_the_notebook_rule():
     assert tm.max() == 64 and tm.dtype == torch.uint8
     # ragged extents are padded with zeros
     fm = torch.ones(2, 130, 9).bool()
-    bm, tm, em = derive_masks(fm)
+    bm, tm, em = O.ref_derive_masks(fm)
     assert bm.shape == (2, 2, 1) and tm.shape == (2, 17, 2) and em.shape == (2, 130, 9)
     assert tm[0, 16, 1] == 2 and tm[0, 0, 0] == 64 and bm.all()
+    # hand-counted: a single kept element, and a kept column that crosses micro-tiles
+    fm = torch.zeros(136, 260, dtype=torch.bool)
+    fm[129, 257] = True
+    fm[3:21, 9] = True
+    bm, tm, em = O.ref_derive_masks(fm)
+    assert bm.tolist() == [[1, 0, 0], [0, 0, 1]]
+    assert int(tm.sum()) == 19 and tm[16, 32] == 1
+    assert [int(tm[i, 1]) for i in range(3)] == [5, 8, 5]
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
