@@ -35,6 +35,7 @@
 // reference (kernels/bmm_helpers.cu:114-164, 240-622).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 
 namespace cmk {
@@ -48,6 +49,8 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef const float __attribute__((address_space(1))) * global_f32_ptr;
 typedef const void __attribute__((address_space(1))) * global_void_ptr;
 typedef void __attribute__((address_space(3))) * lds_void_ptr;
+typedef const float __attribute__((address_space(3))) * lds_f32_ptr;
+typedef const f32x4 __attribute__((address_space(3))) * lds_f32x4_ptr;
 
 constexpr int kThreads = 256;
 // what one (x, y, k) triple contributes to an accumulator
@@ -56,6 +59,15 @@ constexpr int kL2 = 1;      // (x-y)^2, vector unit
 constexpr int kL1 = 2;      // |x-y|,   vector unit
 constexpr int KC = 0;   // k-contiguous operand
 constexpr int RC = 1;   // row-contiguous operand
+
+// f(integral_constant<int, I>) for I = 0 .. N-1, unrolled at compile time.
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
 
 struct Operand {
   const float* p;  // base of this batch's matrix
@@ -123,6 +135,52 @@ __device__ __forceinline__ void lane_offsets_bytes(const Operand& o, int tid,
   }
 }
 
+// One operand's slab -> LDS for a tile that crosses an edge of the matrix or
+// whose operand rules out direct loads: every element is fetched from a clamped
+// (always valid) address, zeroed when it lies outside the matrix, and stored
+// from registers.  A real function on purpose: it runs for edge tiles only, and
+// inlined at every request site it made up most of a kernel's code, which the
+// interior path then had to jump across (instruction-cache misses).
+template <int KIND, int T, int KS, int NT>
+__device__ __noinline__ void fetch_edge(const float* p, long long ld, int rows, int K, int r0,
+                                        int k0, float* dst, int tid) {
+  // NT threads x 4 floats per pass, walking the tile in its memory order
+  constexpr int RUN = KIND == KC ? KS : T;        // contiguous floats per line
+  constexpr int TPR = RUN / 4;                    // threads per line
+  constexpr int LPP = NT / TPR;                   // lines per pass
+  constexpr int LINES = KIND == KC ? T : KS;
+  constexpr int PASSES = (LINES + LPP - 1) / LPP;
+  constexpr bool kAllLines = PASSES * LPP == LINES;  // otherwise some threads have no line
+  const int t = tid;
+  const int c4 = (t % TPR) * 4;
+  f32x4 v[PASSES];
+  const bool any = K > 0 && rows > 0;
+#pragma unroll
+  for (int q = 0; q < PASSES; ++q) {
+    const int line = t / TPR + q * LPP;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int rj = KIND == KC ? r0 + line : r0 + c4 + j;
+      const int kj = KIND == KC ? k0 + c4 + j : k0 + line;
+      const bool ok = any && rj < rows && kj < K && (kAllLines || line < LINES);
+      const long long e = KIND == KC ? (long long)rj * ld + kj : (long long)kj * ld + rj;
+      v[q][j] = any ? *(global_f32_ptr)(ok ? p + e : p) : 0.f;
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < PASSES; ++q) {
+    const int line = t / TPR + q * LPP;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int rj = KIND == KC ? r0 + line : r0 + c4 + j;
+      const int kj = KIND == KC ? k0 + c4 + j : k0 + line;
+      v[q][j] = (rj < rows && kj < K) ? v[q][j] : 0.f;
+    }
+    const int pos = KIND == KC ? lds_pos<KC, T, KS>(line, c4) : lds_pos<RC, T, KS>(c4, line);
+    if (kAllLines || line < LINES) *reinterpret_cast<f32x4*>(dst + pos) = v[q];
+  }
+}
+
 // Work-group level tile engine.  WX x WY waves (4, 8 or 16 of them), each wave owns
 // BX x BY blocks of 32x32; KS is the contraction depth of one LDS slab.
 //
@@ -141,8 +199,11 @@ __device__ __forceinline__ void lane_offsets_bytes(const Operand& o, int tid,
 constexpr int kReadsPaired = 1;   // two-address reads (k, k+1) with immediate offsets, one bank each
 constexpr int kReadsSingle = 2;   // four single reads with immediate offsets
 
+// ADDR_REGS keeps every fragment address in a register of its own for the whole
+// sequence (no vector arithmetic in the slab loop); without it the compiler is
+// free to re-derive them, which a kernel short of registers prefers.
 template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32, int RC_READS = kReadsPaired,
-          bool STAGGER = false, bool Y_ONCE = false>
+          bool STAGGER = false, bool Y_ONCE = false, bool ADDR_REGS = true>
 struct Core {
   static_assert(WX * WY == 4 || WX * WY == 8 || WX * WY == 16, "4, 8 or 16 waves per work-group");
   static constexpr int NT = WX * WY * 64;      // threads per work-group
@@ -169,7 +230,14 @@ struct Core {
   int xbase, y0, K;
   int xr, yr, half, tid;
   int xfast, yfast;          // operand allows direct loads: aligned, offsets fit 32 bits (wave-uniform)
-  int xrow[BX], yrow[BY];    // LDS row of each block; see begin()
+  // LDS byte addresses of this lane's fragments in buffer 0, kept in registers
+  // for the whole sequence so that a fragment read is (register + immediate):
+  // a row-contiguous operand needs one per block (k advances by immediates), a
+  // k-contiguous one needs one per block and k-group (the chunk swizzle is an
+  // exclusive-or, not a sum)
+  static constexpr int NAX = XK == KC ? NG : 1;
+  static constexpr int NAY = YK == KC ? NG : 1;
+  unsigned xad[BX][NAX], yad[BY][NAY];
   unsigned xoff[MX::NV];     // this lane's byte offsets for the direct loads
   unsigned yoff[MY::NV];
   float* pend_buf;           // where the Y slab that is still to be requested goes (wave-uniform)
@@ -180,10 +248,9 @@ struct Core {
   bool late;                 // this wave requests its slabs two k-groups after its SIMD partner
 
   // One operand's slab -> LDS.  Interior tiles: NV direct loads per wave.  Edge
-  // tiles: every element is fetched from a clamped (always valid) address,
-  // zeroed when it lies outside the matrix, and stored from registers.
+  // tiles: fetch_edge().
   template <int KIND, int T, class M>
-  __device__ __forceinline__ void fetch(const Operand& o, const unsigned (&off)[M::NV], int r0,
+  __device__ __forceinline__ void fetch(const Operand& o, unsigned (&off)[M::NV], int r0,
                                         int k0, long long first, float* dst, int fast) {
     // plain integers, so that the test stays in 32-bit scalar registers
     const int interior = fast & static_cast<int>(k0 + KS <= K) & static_cast<int>(r0 + T <= o.rows);
@@ -197,47 +264,15 @@ struct Core {
 #pragma unroll
       for (int p = 0; p < M::NV; ++p)
         if (M::kEven || p * M::NW + wave < M::NI) {
-          unsigned o32 = off[p];
-          asm volatile("" : "+v"(o32));  // keeps the offset a 32-bit register at this point
+          // keeps the offset a 32-bit register at this point; pinned in place, so
+          // that no copy is made
+          asm volatile("" : "+v"(off[p]));
+          const unsigned o32 = off[p];
           __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + o32),
                                            (lds_void_ptr)(dst + (p * M::NW + wave) * 256), 16, 0, 0);
         }
     } else {
-      // NT threads x 4 floats per pass, walking the tile in its memory order
-      constexpr int RUN = KIND == KC ? KS : T;        // contiguous floats per line
-      constexpr int TPR = RUN / 4;                    // threads per line
-      constexpr int LPP = NT / TPR;                   // lines per pass
-      constexpr int LINES = KIND == KC ? T : KS;
-      constexpr int PASSES = (LINES + LPP - 1) / LPP;
-      constexpr bool kAllLines = PASSES * LPP == LINES;  // otherwise some threads have no line
-      const int t = tid;
-      const int c4 = (t % TPR) * 4;
-      f32x4 v[PASSES];
-      const bool any = K > 0 && o.rows > 0;
-#pragma unroll
-      for (int p = 0; p < PASSES; ++p) {
-        const int line = t / TPR + p * LPP;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int rj = KIND == KC ? r0 + line : r0 + c4 + j;
-          const int kj = KIND == KC ? k0 + c4 + j : k0 + line;
-          const bool ok = any && rj < o.rows && kj < K && (kAllLines || line < LINES);
-          const long long e = KIND == KC ? (long long)rj * o.ld + kj : (long long)kj * o.ld + rj;
-          v[p][j] = any ? *(global_f32_ptr)(ok ? o.p + e : o.p) : 0.f;
-        }
-      }
-#pragma unroll
-      for (int p = 0; p < PASSES; ++p) {
-        const int line = t / TPR + p * LPP;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int rj = KIND == KC ? r0 + line : r0 + c4 + j;
-          const int kj = KIND == KC ? k0 + c4 + j : k0 + line;
-          v[p][j] = (rj < o.rows && kj < K) ? v[p][j] : 0.f;
-        }
-        const int pos = KIND == KC ? lds_pos<KC, T, KS>(line, c4) : lds_pos<RC, T, KS>(c4, line);
-        if (kAllLines || line < LINES) *reinterpret_cast<f32x4*>(dst + pos) = v[p];
-      }
+      fetch_edge<KIND, T, KS, NT>(o.p, o.ld, o.rows, K, r0, k0, dst, tid);
     }
   }
 
@@ -273,24 +308,28 @@ struct Core {
     pend_xbuf = nullptr;
   }
 
-  template <int KIND, int T>
-  __device__ __forceinline__ f32x4 frag(const float* lds, int row, int kg) {
+  // Four k values (8*kg + 4*half + 0..3) of one block row of this lane, from the
+  // buffer `off` floats behind buffer 0.  With a compile-time `off` the whole
+  // displacement is an immediate of the read.
+  template <int KIND, int T, int NA>
+  __device__ __forceinline__ f32x4 frag(const unsigned (&ad)[NA], int off, int kg) const {
     if constexpr (KIND == KC) {
-      return *reinterpret_cast<const f32x4*>(&lds[lds_pos<KC, T, KS>(row, kg * 8 + half * 4)]);
+      return *(lds_f32x4_ptr)(ad[kg] + 4u * off);
     } else {
       f32x4 r;
+      const unsigned at = ad[0] + 4u * (off + kg * 8 * T);
       if constexpr (RC_READS == kReadsSingle) {
         // volatile keeps the reads single: 16-bit immediate offsets from one
         // address register
         const volatile float __attribute__((address_space(3)))* q =
-            (const volatile float __attribute__((address_space(3)))*)&lds[(kg * 8 + half * 4) * T + row];
+            (const volatile float __attribute__((address_space(3)))*)at;
         r.x = q[0];
         r.y = q[T];
         r.z = q[2 * T];
         r.w = q[3 * T];
         return r;
       }
-      const float* q = &lds[(kg * 8 + half * 4) * T + row];
+      lds_f32_ptr q = (lds_f32_ptr)at;
       r.x = q[0];
       r.y = q[T];
       r.z = q[2 * T];
@@ -298,13 +337,13 @@ struct Core {
       return r;
     }
   }
-  // Four k values (8*kg + 4*half + 0..3) of every block row of this lane.
-  __device__ __forceinline__ void read_frags(const float* xb, const float* yb, int kg,
-                                             f32x4 (&fx)[BX], f32x4 (&fy)[BY]) {
+  // Fragments of k-group kg from the X buffer at float offset xo and the Y buffer at yo.
+  __device__ __forceinline__ void read_frags(int xo, int yo, int kg,
+                                             f32x4 (&fx)[BX], f32x4 (&fy)[BY]) const {
 #pragma unroll
-    for (int b = 0; b < BX; ++b) fx[b] = frag<XK, TX>(xb, xrow[b], kg);
+    for (int b = 0; b < BX; ++b) fx[b] = frag<XK, TX, NAX>(xad[b], xo, kg);
 #pragma unroll
-    for (int b = 0; b < BY; ++b) fy[b] = frag<YK, TY>(yb, yrow[b], kg);
+    for (int b = 0; b < BY; ++b) fy[b] = frag<YK, TY, NAY>(yad[b], yo, kg);
   }
 
   // Waits until this wave's direct loads have landed in LDS.
@@ -326,20 +365,28 @@ struct Core {
     half = lane >> 5;
     xr = (wave % WX) * BX * 32 + (lane & 31);
     yr = (wave / WX) * BY * 32 + (lane & 31);
-    // The rows of a wave's blocks are 32 apart.  The compiler is not told: it
-    // would fuse the 32-bit column reads of neighbouring blocks into
-    // two-address reads whose 8-bit offsets then need a vector add per pair.
-    // Kept apart, the reads of one block pair up as (k, k+1) with immediate
-    // offsets from one address register.
+    {
+      // Opaque to the compiler, so that the addresses stay in their registers
+      // instead of being re-derived (vector adds cost matrix-pipe time) and so
+      // that reads of neighbouring blocks are not fused into two-address reads
+      // whose 8-bit offsets would need an add per pair.
+      const unsigned base = static_cast<unsigned>(reinterpret_cast<uintptr_t>((lds_f32_ptr)lds));
 #pragma unroll
-    for (int b = 0; b < BX; ++b) {
-      xrow[b] = xr + 32 * b;
-      if (RC_READS == kReadsPaired) asm volatile("" : "+v"(xrow[b]));
-    }
+      for (int b = 0; b < BX; ++b)
 #pragma unroll
-    for (int b = 0; b < BY; ++b) {
-      yrow[b] = yr + 32 * b;
-      if (RC_READS == kReadsPaired) asm volatile("" : "+v"(yrow[b]));
+        for (int g = 0; g < NAX; ++g) {
+          const int row = xr + 32 * b;
+          xad[b][g] = base + 4u * (XK == KC ? lds_pos<KC, TX, KS>(row, g * 8 + half * 4) : half * 4 * TX + row);
+          if (ADDR_REGS) asm volatile("" : "+v"(xad[b][g]));
+        }
+#pragma unroll
+      for (int b = 0; b < BY; ++b)
+#pragma unroll
+        for (int g = 0; g < NAY; ++g) {
+          const int row = yr + 32 * b;
+          yad[b][g] = base + 4u * (YK == KC ? lds_pos<KC, TY, KS>(row, g * 8 + half * 4) : half * 4 * TY + row);
+          if (ADDR_REGS) asm volatile("" : "+v"(yad[b][g]));
+        }
     }
     xbase = __builtin_amdgcn_readfirstlane(xbase_);
     y0 = __builtin_amdgcn_readfirstlane(y0_);
@@ -379,25 +426,45 @@ struct Core {
     wait_loads();
     __syncthreads();
     if (iters > 1) issue_x(X, xbuf(lds, 1));
-    read_frags(lds, ybuf(lds, 0, 0), 0, xf[0], yf[0]);
+    read_frags(xoff_of(0), yoff_of(0, 0), 0, xf[0], yf[0]);
   }
 
   // LDS buffers of flat slab `i`, whose k-slab index is `s`.  Without Y_ONCE an
   // X and a Y slab sit side by side, twice; with it, two X buffers are followed
   // by two Y buffers that alternate with the k-slab.
-  __device__ __forceinline__ float* xbuf(float* lds, int i) const {
-    return lds + (i & 1) * (Y_ONCE ? xFloats : bufFloats);
+  __device__ __forceinline__ int xoff_of(int i) const {
+    return (i & 1) * (Y_ONCE ? xFloats : bufFloats);
   }
-  __device__ __forceinline__ float* ybuf(float* lds, int i, int s) const {
-    return Y_ONCE ? lds + 2 * xFloats + (s & 1) * yFloats : xbuf(lds, i) + xFloats;
+  __device__ __forceinline__ int yoff_of(int i, int s) const {
+    return Y_ONCE ? 2 * xFloats + (s & 1) * yFloats : xoff_of(i) + xFloats;
   }
+  __device__ __forceinline__ float* xbuf(float* lds, int i) const { return lds + xoff_of(i); }
+  __device__ __forceinline__ float* ybuf(float* lds, int i, int s) const { return lds + yoff_of(i, s); }
 
   // acc += the current tile's product: S slabs of the flat sequence.
-  template <int DIST = kInner>
+  // With FRESH the accumulators need no clearing: the tile's first matrix
+  // instructions take a literal zero as their addend, which saves the 16 * BX * BY
+  // vector moves that would otherwise stall the matrix pipe.
+  template <int DIST = kInner, bool FRESH = false>
   __device__ __forceinline__ void tile(const Operand& X, const Operand& Y, float* lds,
                                        f32x16 (&acc)[BX][BY]) {
     static_assert(!Y_ONCE, "with Y_ONCE the kernel walks slabs itself: tiles inside k-slabs");
-    for (int s = 0; s < S; ++s) slab<DIST>(X, Y, lds, acc);
+    static_assert(!FRESH || DIST == kInner, "only the matrix path can start from a literal zero");
+    if constexpr (DIST != kInner) {
+      for (int s = 0; s < S; ++s) slab<DIST>(X, Y, lds, acc);
+    } else if ((S & 1) == 0) {
+      // an even slab count keeps the flat slab counter even at every tile
+      // start: the buffer of each slab is then known at compile time
+      slab<DIST, FRESH, 0>(X, Y, lds, acc);
+      slab<DIST, false, 1>(X, Y, lds, acc);
+      for (int s = 2; s < S; s += 2) {
+        slab<DIST, false, 0>(X, Y, lds, acc);
+        slab<DIST, false, 1>(X, Y, lds, acc);
+      }
+    } else {
+      slab<DIST, FRESH>(X, Y, lds, acc);
+      for (int s = 1; s < S; ++s) slab<DIST>(X, Y, lds, acc);
+    }
   }
 
   // The distances other than the inner product have no matrix-pipe form.  They
@@ -465,7 +532,12 @@ struct Core {
   }
 
   // acc += one slab of the flat sequence.
-  template <int DIST = kInner>
+  // PAR >= 0 states the parity of the flat slab counter, i.e. which X buffer
+  // (and, without Y_ONCE, which Y buffer) the slab lives in, at compile time:
+  // fragment reads then need no address arithmetic at all.
+  // With Y_ONCE the Y buffer alternates with the k-slab instead: YPAR / YNPAR
+  // state the k-slab parity of this slab and of the next one in the sequence.
+  template <int DIST = kInner, bool FRESH = false, int PAR = -1, int YPAR = -1, int YNPAR = -1>
   __device__ __forceinline__ void slab(const Operand& X, const Operand& Y, float* lds,
                                        f32x16 (&acc)[BX][BY]) {
     if constexpr (DIST != kInner) {
@@ -485,11 +557,12 @@ struct Core {
       ++it;
       if (Y_ONCE && ++ct == nt) { ct = 0; ++cs; }
     } else {
-      float* cur = xbuf(lds, it);
-      const float* nxt = xbuf(lds, it + 1);
       const int ns = (Y_ONCE && ct + 1 == nt) ? cs + 1 : cs;   // k-slab of the next flat slab
-      const float* ycur = ybuf(lds, it, cs);
-      const float* ynxt = ybuf(lds, it + 1, ns);
+      const int curx = xoff_of(PAR < 0 ? it : PAR);
+      const int nxtx = xoff_of(PAR < 0 ? it + 1 : PAR + 1);
+      const int cury = (Y_ONCE && YPAR >= 0) ? yoff_of(0, YPAR) : yoff_of(PAR < 0 ? it : PAR, cs);
+      const int nxty = (Y_ONCE && YNPAR >= 0) ? yoff_of(0, YNPAR) : yoff_of(PAR < 0 ? it + 1 : PAR + 1, ns);
+      float* cur = lds + curx;
       const bool has1 = it + 1 < iters;
       const bool has2 = it + 2 < iters;
 #pragma unroll
@@ -501,19 +574,19 @@ struct Core {
 #pragma unroll
           for (int by = 0; by < BY; ++by)
             acc[bx][by] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                xf[kg & 1][bx][0], yf[kg & 1][by][0], acc[bx][by], 0, 0, 0);
+                xf[kg & 1][bx][0], yf[kg & 1][by][0], (FRESH && kg == 0) ? f32x16{} : acc[bx][by], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (kg == 0 && !late) issue_y(Y);
         if (kg == 1 && late) issue_pending_x(X);
         if (kg == 2 && late) issue_y(Y);
         if (kg + 1 < NG) {
-          read_frags(cur, ycur, kg + 1, xf[(kg + 1) & 1], yf[(kg + 1) & 1]);
+          read_frags(curx, cury, kg + 1, xf[(kg + 1) & 1], yf[(kg + 1) & 1]);
         } else if (has1) {
           wait_loads();     // this wave's part of slab it+1 is in LDS
           __syncthreads();  // everyone's is, and nobody reads `cur` any more
           pend_xbuf = has2 ? cur : nullptr;
           if (!late) issue_pending_x(X);
-          read_frags(nxt, ynxt, 0, xf[0], yf[0]);
+          read_frags(nxtx, nxty, 0, xf[0], yf[0]);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll

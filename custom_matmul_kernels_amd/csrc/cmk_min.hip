@@ -72,13 +72,15 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
   core.begin(X, Y, xt_begin * C::TX, y0, a.K, xt_end - xt_begin, lds);
   for (int xt = xt_begin; xt < xt_end; ++xt) {
     f32x16 acc[2][2];
+    if constexpr (DIST != kInner) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    core.template tile<DIST>(X, Y, lds, acc);
+          for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    }
+    core.template tile<DIST, DIST == kInner>(X, Y, lds, acc);
     // fold this tile into the running minimum; indices ascend within a lane,
     // so a strict '<' keeps the first occurrence
     const int xb = xt * C::TX + wx * 64;

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   constexpr int kBX = MULTI ? 1 : 2;
   constexpr int kTX = kTileX * kBX;             // candidates per tile in this kernel
   constexpr int kCT = kChunkTiles / kBX;        // tiles per chunk in this kernel
-  using C = Core<XK, YK, 8, 2, kBX, 1, 32, kReadsSingle, false, true>;
+  using C = Core<XK, YK, 8, 2, kBX, 1, 32, kReadsSingle, false, true, false>;
   static_assert(C::TX == kTX && C::TY == kStripRows && C::NT == kTopkThreads, "tile shape");
   // LDS: operand buffers, reused as the staging area; the lists follow the
   // staging area (MULTI: the operand buffers, which they must outlive)
@@ -102,14 +102,14 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
     __syncthreads();  // previous chunk's staging reads are finished
     core.begin(X, Y, xt0 * kTileX, y0, a.K, nt, lds);
     f32x16 acc[kCT][kBX][1];
+    // k-slabs outside, tiles inside: a slab of the strip's own rows is fetched
+    // once and meets the chunk's tiles one after the other
 #pragma unroll
     for (int i = 0; i < kCT; ++i)
 #pragma unroll
       for (int bx = 0; bx < kBX; ++bx)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][bx][0][r] = 0.f;
-    // k-slabs outside, tiles inside: a slab of the strip's own rows is fetched
-    // once and meets the chunk's tiles one after the other
     for (int s = 0; s < core.S; ++s) {
 #pragma unroll
       for (int i = 0; i < kCT; ++i)
