@@ -246,6 +246,7 @@ struct Core {
   long long pend_y;          // and its element offset
   float* pend_xbuf;          // buffer whose X half is still to be requested (wave-uniform)
   bool late;                 // this wave requests its slabs two k-groups after its SIMD partner
+  int wave_s;                // ADDR_REGS: the wave's index, kept in a scalar register
 
   // One operand's slab -> LDS.  Interior tiles: NV direct loads per wave.  Edge
   // tiles: fetch_edge().
@@ -254,19 +255,24 @@ struct Core {
                                         int k0, long long first, float* dst, int fast) {
     // plain integers, so that the test stays in 32-bit scalar registers
     const int interior = fast & static_cast<int>(k0 + KS <= K) & static_cast<int>(r0 + T <= o.rows);
+    // Keeps each offset a plain 32-bit register where the loads use it (the load
+    // is then scalar base + lane offset).  Pinned in place and ahead of the
+    // branch: no copies, and both paths leave the same registers behind.
+    if constexpr (ADDR_REGS) {
+#pragma unroll
+      for (int p = 0; p < M::NV; ++p) asm volatile("" : "+v"(off[p]));
+    }
     if (interior) {
       // the tile's address is the same in every lane; pinned to scalar registers
       // so that each load is (scalar base + 32-bit lane offset) with no vector add
       unsigned long long tile_bits = reinterpret_cast<unsigned long long>(o.p + first);
       asm volatile("" : "+s"(tile_bits));
       const char* tile = reinterpret_cast<const char*>(tile_bits);
-      const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+      const int wave = ADDR_REGS ? wave_s : __builtin_amdgcn_readfirstlane(tid >> 6);
 #pragma unroll
       for (int p = 0; p < M::NV; ++p)
         if (M::kEven || p * M::NW + wave < M::NI) {
-          // keeps the offset a 32-bit register at this point; pinned in place, so
-          // that no copy is made
-          asm volatile("" : "+v"(off[p]));
+          if constexpr (!ADDR_REGS) asm volatile("" : "+v"(off[p]));  // short of registers: pinned where used
           const unsigned o32 = off[p];
           __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + o32),
                                            (lds_void_ptr)(dst + (p * M::NW + wave) * 256), 16, 0, 0);
@@ -363,6 +369,7 @@ struct Core {
     const int lane = tid & 63;
     const int wave = tid >> 6;
     half = lane >> 5;
+    wave_s = __builtin_amdgcn_readfirstlane(wave);
     xr = (wave % WX) * BX * 32 + (lane & 31);
     yr = (wave / WX) * BY * 32 + (lane & 31);
     {
