@@ -229,7 +229,10 @@ struct Core {
   long long xrun, yrun, xstep_in, xstep_out, ystep;
   int xbase, y0, K;
   int xr, yr, half, tid;
-  int xfast, yfast;          // operand allows direct loads: aligned, offsets fit 32 bits (wave-uniform)
+  // Interior test of a slab in three scalar subtractions: last first-row (and
+  // last first-k) at which a whole tile still lies inside the matrix; -1 for an
+  // operand that rules out direct loads (unaligned, or offsets beyond 32 bits).
+  int xlast, ylast, klast;
   // LDS byte addresses of this lane's fragments in buffer 0, kept in registers
   // for the whole sequence so that a fragment read is (register + immediate):
   // a row-contiguous operand needs one per block (k advances by immediates), a
@@ -252,9 +255,10 @@ struct Core {
   // tiles: fetch_edge().
   template <int KIND, int T, class M>
   __device__ __forceinline__ void fetch(const Operand& o, unsigned (&off)[M::NV], int r0,
-                                        int k0, long long first, float* dst, int fast) {
-    // plain integers, so that the test stays in 32-bit scalar registers
-    const int interior = fast & static_cast<int>(k0 + KS <= K) & static_cast<int>(r0 + T <= o.rows);
+                                        int k0, long long first, float* dst, int rlast) {
+    // both differences are non-negative exactly for an interior slab; one sign
+    // test on plain 32-bit scalars
+    const bool interior = ((klast - k0) | (rlast - r0)) >= 0;
     // Keeps each offset a plain 32-bit register where the loads use it (the load
     // is then scalar base + lane offset).  Pinned in place and ahead of the
     // branch: no copies, and both paths leave the same registers behind.
@@ -290,7 +294,7 @@ struct Core {
     // address arithmetic on the scalar unit
     const int x0 = __builtin_amdgcn_readfirstlane(xbase + lt * TX);
     pend_k0 = __builtin_amdgcn_readfirstlane(ls * KS);
-    fetch<XK, TX, MX>(X, xoff, x0, pend_k0, xrun, buf, xfast);
+    fetch<XK, TX, MX>(X, xoff, x0, pend_k0, xrun, buf, xlast);
     if constexpr (Y_ONCE) {
       // tiles run inside slabs: the Y slab is fetched with the first tile only
       pend_buf = lt == 0 ? ybase + (ls & 1) * yFloats : nullptr;
@@ -306,7 +310,7 @@ struct Core {
     }
   }
   __device__ __forceinline__ void issue_y(const Operand& Y) {
-    if (pend_buf) fetch<YK, TY, MY>(Y, yoff, y0, pend_k0, pend_y, pend_buf, yfast);
+    if (pend_buf) fetch<YK, TY, MY>(Y, yoff, y0, pend_k0, pend_y, pend_buf, ylast);
     pend_buf = nullptr;
   }
   __device__ __forceinline__ void issue_pending_x(const Operand& X) {
@@ -399,8 +403,9 @@ struct Core {
     y0 = __builtin_amdgcn_readfirstlane(y0_);
     K = __builtin_amdgcn_readfirstlane(K_);
     S = max(1, (K + KS - 1) / KS);
-    xfast = X.vec != 0 && (long long)(TX + KS) * X.ld < (1ll << 29);
-    yfast = Y.vec != 0 && (long long)(TY + KS) * Y.ld < (1ll << 29);
+    xlast = (X.vec != 0 && (long long)(TX + KS) * X.ld < (1ll << 29)) ? X.rows - TX : -1;
+    ylast = (Y.vec != 0 && (long long)(TY + KS) * Y.ld < (1ll << 29)) ? Y.rows - TY : -1;
+    klast = K - KS;
     nt = __builtin_amdgcn_readfirstlane(ntiles);
     iters = nt * S;
     ct = 0;
