@@ -219,7 +219,7 @@ def main():
     if a.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported "
               "(every output row depends on one row of A and all of B, so the path "
-              "shards by rows without communication; see DESIGN.md)" % a.gpus, file=sys.stderr)
+              "would shard by rows without communication)" % a.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch
