@@ -170,22 +170,34 @@ __global__ void min_fold_kernel(const float* part_val, const int* part_idx, floa
   indices[i] = idx;
 }
 
-// How the work is cut.  The reduced axis is split (a) when the kept axis alone
-// does not give every CU a couple of work-groups and (b) when X is too large
-// to stay in an XCD's L2, so that fewer distinct Y strips are live per XCD.
+// How the work is cut.  Splitting the reduced axis gives more work-groups than
+// the kept axis alone has strips; every candidate split count is priced as
+// (rounds the machine needs for all work-groups, two per CU) x (slabs one
+// work-group multiplies + a fixed cost for filling the pipeline and folding) and
+// the cheapest is taken.  When X is too large to stay in an XCD's L2 at least
+// four splits are used, so that fewer distinct Y strips are live per XCD.
 static void plan_min(int L, int Xext, int Yext, int K, int* ystrips, int* xtiles, int* splits,
                      int* tiles_per_split, int* ygroup) {
   *ystrips = ceil_div(Yext, 128);
   *xtiles = ceil_div(Xext, 128);
   const long long strips = (long long)L * *ystrips;
-  int want = 1;
-  if (strips < 512) want = (int)((512 + strips - 1) / strips);
-  if ((long long)Xext * K * 4 > (2ll << 20) && *xtiles >= 32 && want < 4) want = 4;
-  if (want > *xtiles) want = *xtiles;
-  if (want > 64) want = 64;
-  if (want < 1) want = 1;
-  *tiles_per_split = ceil_div(*xtiles, want);
-  *splits = ceil_div(*xtiles, *tiles_per_split);
+  const long long slots = 2ll * compute_units();
+  const long long slabs = K > 0 ? ceil_div(K, 32) : 1;
+  const bool big_x = (long long)Xext * K * 4 > (2ll << 20) && *xtiles >= 32;
+  const int most = *xtiles < 64 ? *xtiles : 64;
+  long long best_cost = -1;
+  int best_tps = *xtiles > 0 ? *xtiles : 1;
+  for (int want = big_x ? 4 : 1; want <= most; ++want) {
+    const int tps = ceil_div(*xtiles, want);
+    const int s = ceil_div(*xtiles, tps);
+    const int yg = 64 / s > 0 ? 64 / s : 1;
+    const long long total = ((strips + yg - 1) / yg) * yg * s;
+    const long long rounds = (total + slots - 1) / slots;
+    const long long cost = rounds * (tps * slabs + 6);
+    if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_tps = tps; }
+  }
+  *tiles_per_split = best_tps;
+  *splits = *xtiles > 0 ? ceil_div(*xtiles, best_tps) : 1;
   *ygroup = 64 / *splits > 0 ? 64 / *splits : 1;
 }
 
