@@ -430,8 +430,8 @@ struct Core {
     pend_xbuf = nullptr;
     // STAGGER: the upper half of the waves does its address arithmetic and load
     // requests two k-groups after the lower half, which spreads the requests
-    // over the slab (measured: a gain for the 4-wave min kernel, a loss for the
-    // 8-wave top-k kernel)
+    // over the slab (measured: a gain for the 4-wave min kernel, none for the
+    // top-k kernel)
     late = STAGGER && __builtin_amdgcn_readfirstlane(wave) >= WX * WY / 2;
     issue_x(X, lds);
     issue_y(Y);

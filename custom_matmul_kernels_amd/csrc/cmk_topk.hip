@@ -175,7 +175,7 @@ extern "C" int cmk_topk_bmm_f32(const float* A, const float* B, float* values, l
   }
   const long long total = (long long)d->L * a.ystrips * a.splits;
   if (int e = check_grid(total)) return e;
-  // one eight-wave work-group per CU is resident at a time; two per CU even out the tail
+  // one sixteen-wave work-group per CU is resident at a time; a grid of two per CU evens out the tail
   const long long padded = ((total + 7) / 8) * 8;
   const long long machine = 2ll * compute_units();
   const dim3 grid((unsigned)(padded < machine ? padded : machine)), block(kTopkThreads);
