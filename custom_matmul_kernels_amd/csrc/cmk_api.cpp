@@ -61,7 +61,7 @@ int compute_units() {
 }
 
 size_t min_workspace_bytes(int L, int Xext, int Yext, int K);
-size_t topk_workspace_bytes(int L, int Xext, int Yext);
+size_t topk_workspace_bytes(int L, int Xext, int Yext, int K);
 size_t topk1d_workspace_bytes(long long n);
 
 }  // namespace cmk
@@ -74,7 +74,7 @@ extern "C" size_t cmk_workspace_bytes(int op, int L, int M, int N, int K, int di
       return cmk::min_workspace_bytes(L, dim == 2 ? N : M, dim == 2 ? M : N, K);
     case CMK_OP_TOPK_BMM:
       if (dim != 1 && dim != 2) return 0;
-      return cmk::topk_workspace_bytes(L, dim == 2 ? N : M, dim == 2 ? M : N);
+      return cmk::topk_workspace_bytes(L, dim == 2 ? N : M, dim == 2 ? M : N, K);
     case CMK_OP_TOPK_1D:
       return cmk::topk1d_workspace_bytes(M);
     default:

@@ -95,24 +95,35 @@ __global__ __launch_bounds__(kThreads) void topk1d_partial_kernel(const float* a
   part[o + lane + 64] = list[wave][lane + 64];
 }
 
-static void plan_topk(int L, int Xext, int Yext, int* ystrips, int* xtiles, int* splits,
+static void plan_topk(int L, int Xext, int Yext, int K, int* ystrips, int* xtiles, int* splits,
                       int* tiles_per_split) {
   *ystrips = ceil_div(Yext, kStripRows);
   *xtiles = ceil_div(Xext, kTileX);
   const long long strips = (long long)L * *ystrips;
   const int chunks = ceil_div(*xtiles, kChunkTiles);
-  int want = 1;
-  if (strips < 256) want = (int)((256 + strips - 1) / strips);
-  if (want > chunks) want = chunks;
-  if (want < 1) want = 1;
-  const int chunks_per_split = ceil_div(chunks, want);
-  *tiles_per_split = chunks_per_split * kChunkTiles;
-  *splits = ceil_div(*xtiles, *tiles_per_split);
+  // Every candidate split count is priced as (rounds the machine needs, one
+  // work-group per CU) x (chunks per work-group x (slabs of a chunk + its
+  // selection, worth about 3.5 slabs) + ordering and start-up), plus the merge
+  // launch when the reduced axis is split; the cheapest wins.
+  const long long slots = compute_units();
+  const long long slabs = K > 0 ? ceil_div(K, 32) : 1;
+  const int most = chunks < 64 ? chunks : 64;
+  long long best_cost = -1;
+  int best_cps = chunks > 0 ? chunks : 1;
+  for (int want = 1; want <= most; ++want) {
+    const int cps = ceil_div(chunks, want);
+    const int s = ceil_div(chunks, cps);
+    const long long rounds = (strips * s + slots - 1) / slots;
+    const long long cost = rounds * (cps * (2 * slabs + 7) + 4) + (s > 1 ? 3 : 0);   // in half slabs
+    if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_cps = cps; }
+  }
+  *tiles_per_split = best_cps * kChunkTiles;
+  *splits = *xtiles > 0 ? ceil_div(*xtiles, *tiles_per_split) : 1;
 }
 
-size_t topk_workspace_bytes(int L, int Xext, int Yext) {
+size_t topk_workspace_bytes(int L, int Xext, int Yext, int K) {
   int ys, xt, sp, tps;
-  plan_topk(L, Xext, Yext, &ys, &xt, &sp, &tps);
+  plan_topk(L, Xext, Yext, K, &ys, &xt, &sp, &tps);
   if (sp <= 1) return 0;
   return (size_t)sp * L * Yext * kTop * 8;
 }
@@ -164,7 +175,7 @@ extern "C" int cmk_topk_bmm_f32(const float* A, const float* B, float* values, l
   a.L = d->L;
   a.K = d->K;
   a.k = k;
-  plan_topk(d->L, Xext, Yext, &a.ystrips, &a.xtiles, &a.splits, &a.tiles_per_split);
+  plan_topk(d->L, Xext, Yext, d->K, &a.ystrips, &a.xtiles, &a.splits, &a.tiles_per_split);
   if (a.xtiles == 0) { a.xtiles = 0; a.splits = 1; a.tiles_per_split = kChunkTiles; }
   if (a.splits > 1) {
     const size_t need = (size_t)a.splits * d->L * Yext * kTop * 8;
