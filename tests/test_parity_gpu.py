@@ -209,6 +209,34 @@ def test_mbmm_mask_precedence_and_integer_exactness(device):
     assert (MBMMCUDA()(A.to(device), B.to(device), zb, ones[1], ones[2]) == 0).all()
 
 
+def test_mbmm_config_3_properties(device):
+    """A[128,1024,64] @ B[128,64,1024] under tril AND tile-Bernoulli(0.5) masks, at
+    full size: dropped elements are exactly zero, kept elements equal the dense
+    product of the same library bit for bit, three batches are checked against
+    float64, and a skipped tile never touches its operands (NaNs planted there
+    do not leak)."""
+    say("mbmm config 3")
+    L, M, N, K = 128, 1024, 1024, 64
+    A, B = seeded(L, M, N, K, seed=0)
+    fm = random_masks(L, M, N, seed=1, share=False)
+    Ad, Bd, fd = A.to(device), B.to(device), fm.to(device)
+    bm, tm, em = derive_masks(fd)
+    C = MBMMCUDA(share_mask=False)(Ad, Bd, bm, tm, em)
+    assert (C[~fd] == 0).all()
+    dense = BMMCUDA()(Ad, Bd)
+    assert torch.equal(C[fd], dense[fd])
+    for b in (0, 77, 127):
+        want = (A[b].double() @ B[b].double()).float() * fm[b]
+        O.check_values(C[b].cpu(), want, K, "mbmm batch %d" % b)
+    # batch 5, tile row 0: rows 0..127 of A feed only tiles (0, 0) (tril); if that
+    # tile is skipped, NaNs in those rows must not show anywhere in the output
+    if bm[5, 0, 0] == 0:
+        A2 = Ad.clone()
+        A2[5, :128] = float("nan")
+        C2 = MBMMCUDA(share_mask=False)(A2, Bd, bm, tm, em)
+        assert torch.equal(C2[5], C[5])
+
+
 # ---------------------------------------------------------------- min_bmm ----
 MIN_SHAPES = [(1, 1, 1, 1), (2, 37, 300, 19), (1, 129, 257, 33), (3, 128, 128, 64),
               (1, 200, 1000, 70), (1, 1000, 200, 12), (2, 64, 2000, 32)]
