@@ -324,7 +324,7 @@ struct Core {
   template <int KIND, int T, int NA>
   __device__ __forceinline__ f32x4 frag(const unsigned (&ad)[NA], int off, int kg) const {
     if constexpr (KIND == KC) {
-      return *(lds_f32x4_ptr)(ad[kg] + 4u * off);
+      return *(lds_f32x4_ptr)static_cast<uintptr_t>(ad[kg] + 4u * off);
     } else {
       f32x4 r;
       const unsigned at = ad[0] + 4u * (off + kg * 8 * T);
@@ -332,14 +332,14 @@ struct Core {
         // volatile keeps the reads single: 16-bit immediate offsets from one
         // address register
         const volatile float __attribute__((address_space(3)))* q =
-            (const volatile float __attribute__((address_space(3)))*)at;
+            (const volatile float __attribute__((address_space(3)))*)static_cast<uintptr_t>(at);
         r.x = q[0];
         r.y = q[T];
         r.z = q[2 * T];
         r.w = q[3 * T];
         return r;
       }
-      lds_f32_ptr q = (lds_f32_ptr)at;
+      lds_f32_ptr q = (lds_f32_ptr)static_cast<uintptr_t>(at);
       r.x = q[0];
       r.y = q[T];
       r.z = q[2 * T];
