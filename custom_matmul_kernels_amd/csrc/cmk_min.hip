@@ -155,16 +155,29 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
 }
 
 // Folds the per-split partial results in ascending split (= ascending index)
-// order.
-__global__ void min_fold_kernel(const float* part_val, const int* part_idx, float* values,
-                                long long* indices, long long rows, int splits) {
+// order.  The partials of eight splits are requested together, so that the
+// kernel waits for memory once per eight splits instead of once per split; 64
+// threads per work-group spread a small problem over more CUs.
+constexpr int kFoldThreads = 64;
+__global__ __launch_bounds__(kFoldThreads) void min_fold_kernel(const float* part_val, const int* part_idx,
+                                                                float* values, long long* indices,
+                                                                long long rows, int splits) {
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= rows) return;
-  float v = part_val[i];
+  float v = INFINITY;
   int idx = part_idx[i];
-  for (int s = 1; s < splits; ++s) {
-    const float ov = part_val[(long long)s * rows + i];
-    if (ov < v) { v = ov; idx = part_idx[(long long)s * rows + i]; }
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float pv[8];
+    int pi[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int s = s0 + j < splits ? s0 + j : splits - 1;   // clamped: repeats fold to nothing
+      pv[j] = part_val[(long long)s * rows + i];
+      pi[j] = part_idx[(long long)s * rows + i];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (pv[j] < v) { v = pv[j]; idx = pi[j]; }
   }
   values[i] = v;
   indices[i] = idx;
@@ -270,7 +283,8 @@ extern "C" int cmk_min_bmm_f32(const float* A, const float* B, float* values, lo
   if (int e = hip_status(hipGetLastError(), "cmk_min_bmm_f32 launch")) return e;
   if (a.splits > 1) {
     const long long rows = (long long)d->L * Yext;
-    hipLaunchKernelGGL(min_fold_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st,
+    hipLaunchKernelGGL(min_fold_kernel, dim3((unsigned)((rows + kFoldThreads - 1) / kFoldThreads)),
+                       dim3(kFoldThreads), 0, st,
                        a.part_val, a.part_idx, values, indices, rows, a.splits);
     if (int e = hip_status(hipGetLastError(), "cmk_min_bmm_f32 fold launch")) return e;
   }
