@@ -104,13 +104,26 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
     f32x16 acc[kCT][kBX][1];
     // k-slabs outside, tiles inside: a slab of the strip's own rows is fetched
     // once and meets the chunk's tiles one after the other
+    // The first k-slab starts the accumulators from a literal zero (matrix path):
+    // no clearing.  Tiles a short last chunk does not have are cleared instead.
+    static_for<0, kCT>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      if (i < nt) {
+        if constexpr (DIST != kInner) {
 #pragma unroll
-    for (int i = 0; i < kCT; ++i)
+          for (int bx = 0; bx < kBX; ++bx)
 #pragma unroll
-      for (int bx = 0; bx < kBX; ++bx)
+            for (int r = 0; r < 16; ++r) acc[i][bx][0][r] = 0.f;
+        }
+        core.template slab<DIST, DIST == kInner>(X, Y, lds, acc[i]);
+      } else {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][bx][0][r] = 0.f;
-    for (int s = 0; s < core.S; ++s) {
+        for (int bx = 0; bx < kBX; ++bx)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][bx][0][r] = 0.f;
+      }
+    });
+    for (int s = 1; s < core.S; ++s) {
 #pragma unroll
       for (int i = 0; i < kCT; ++i)
         if (i < nt) core.template slab<DIST>(X, Y, lds, acc[i]);
