@@ -31,7 +31,7 @@ PEAK_VALU_TOPS = 39.3           # 256 CUs x 64 lanes x 2.4 GHz: one fp32 vector 
 # from inside this process; the figures are those of the summaries in profiles/.
 MEASURED_TRAFFIC_BYTES = {
     "min_bmm_large": (2 * 2.15038e6 + 2048) * 1024,      # profiles/min_kernel_min_bmm_large.txt
-    "topk_bmm": (2 * 882311 + 1.71003e6) * 1024,           # profiles/topk_kernel_topk_bmm.txt
+    "topk_bmm": (2 * 882558 + 1.71006e6) * 1024,           # profiles/topk_kernel_topk_bmm.txt
     "derive_masks_4GiB": (2 * 2.09726e6 + 66564.6) * 1024,  # profiles/derive_masks_kernel_4GiB.txt
 }
 
