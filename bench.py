@@ -194,8 +194,21 @@ def cpu_baseline(torch, wl, args_dev, budget_s=12.0):
     return {"value": round(gflops, 2), "unit": "GFLOP/s", "cores": torch.get_num_threads(),
             "kind": "port",
             "sample": "%s on %d rows in slabs of %d (%.2f passes over the workload's %d rows), "
-                      "%d threads, %.2f s" % (wl["cpu_expr"], done_rows, rows, done_rows / wl["rows"],
-                                              wl["rows"], torch.get_num_threads(), t_total)}
+                      "%d threads of %d logical CPUs (%s), %.2f s"
+                      % (wl["cpu_expr"], done_rows, rows, done_rows / wl["rows"], wl["rows"],
+                         torch.get_num_threads(), os.cpu_count() or 0, cpu_model(), t_total)}
+
+
+def cpu_model():
+    """The host CPU's model string, from /proc/cpuinfo."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown CPU"
 
 
 def run_workload(torch, wl, steps, warmup):
