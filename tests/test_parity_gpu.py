@@ -554,3 +554,40 @@ def test_entry_points_replay_in_a_hip_graph(device):
         torch.cuda.synchronize()
         for g, w in zip(got, want):
             assert torch.equal(g, w), "replay %d differs from the eager result" % step
+
+
+def test_two_host_threads_on_two_streams(device):
+    """The library keeps no state between calls except the thread-local error
+    string: two host threads, each on a stream of its own, get the results they
+    get when run one after the other."""
+    import threading
+    say("host threads")
+    gen = torch.Generator().manual_seed(33)
+    inputs = [(torch.randn(1, 700, 96, generator=gen).to(device), torch.randn(1, 96, 900, generator=gen).to(device))
+              for _ in range(2)]
+    want = [(MinBMMCUDA()(a, b, dim=2), TopkBMMCUDA()(a, b, k=64, dim=2)) for a, b in inputs]
+    torch.cuda.synchronize()
+    got = [None, None]
+    errors = []
+
+    def work(i):
+        try:
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                a, b = inputs[i]
+                for _ in range(20):
+                    r = (MinBMMCUDA()(a, b, dim=2), TopkBMMCUDA()(a, b, k=64, dim=2))
+                s.synchronize()
+                got[i] = r
+        except Exception as e:  # noqa: BLE001 - reported below
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(2):
+        for (gv, gi), (wv, wi) in zip(got[i], want[i]):
+            assert torch.equal(gv, wv) and torch.equal(gi, wi)
