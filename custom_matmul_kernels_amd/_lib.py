@@ -26,6 +26,7 @@ EXPORTS = (
     "cmk_mbmm_f32",
     "cmk_derive_masks_u8",
     "cmk_min_bmm_f32",
+    "cmk_min_bmm_f32_static",
     "cmk_topk_bmm_f32",
     "cmk_topk_1d_f32",
     "cmk_workspace_bytes",
@@ -93,10 +94,11 @@ def load():
     lib.cmk_mbmm_f32.argtypes = [p, p, p, p, p, p, i, dp, p]
     lib.cmk_derive_masks_u8.argtypes = [p, p, p, i, i, i, p]
     lib.cmk_min_bmm_f32.argtypes = [p, p, p, p, dp, i, i, p, sz, p]
+    lib.cmk_min_bmm_f32_static.argtypes = [p, p, p, p, dp, i, i, p]
     lib.cmk_topk_bmm_f32.argtypes = [p, p, p, p, dp, i, i, i, p, sz, p]
     lib.cmk_topk_1d_f32.argtypes = [p, ll, p, p, i, p, sz, p]
-    for name in ("cmk_bmm_f32", "cmk_mbmm_f32", "cmk_derive_masks_u8", "cmk_min_bmm_f32", "cmk_topk_bmm_f32",
-                 "cmk_topk_1d_f32"):
+    for name in ("cmk_bmm_f32", "cmk_mbmm_f32", "cmk_derive_masks_u8", "cmk_min_bmm_f32", "cmk_min_bmm_f32_static",
+                 "cmk_topk_bmm_f32", "cmk_topk_1d_f32"):
         getattr(lib, name).restype = i
     lib.cmk_workspace_bytes.argtypes = [i, i, i, i, i, i]
     lib.cmk_workspace_bytes.restype = sz

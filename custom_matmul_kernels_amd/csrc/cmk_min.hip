@@ -14,6 +14,8 @@
 // atomicMin (reference kernels/minbmm.cu:1-153, 347-440).
 #include <math.h>
 
+#include <atomic>
+
 #include "cmk_core.hpp"
 #include "cmk_launch.hpp"
 
@@ -225,9 +227,12 @@ size_t min_workspace_bytes(int L, int Xext, int Yext, int K) {
 
 using namespace cmk;
 
-extern "C" int cmk_min_bmm_f32(const float* A, const float* B, float* values, long long* indices,
-                               const cmk_gemm_desc* d, int dim, int distance, void* workspace,
-                               size_t workspace_bytes, void* stream) {
+// Validates, plans and enqueues one min_bmm; `workspace` is whatever device
+// memory holds the per-split partial results (the caller's buffer, or the
+// library's static scratch array).
+static int min_bmm_enqueue(const float* A, const float* B, float* values, long long* indices,
+                           const cmk_gemm_desc* d, int dim, int distance, void* workspace,
+                           size_t workspace_bytes, void* stream) {
   if (int e = check_desc(d)) return e;
   if (dim != 1 && dim != 2) return fail(CMK_ERR_INVALID_ARG, "cmk_min_bmm_f32: dim must be 1 or 2");
   if (distance < CMK_DIST_INNER || distance > CMK_DIST_L1)
@@ -289,4 +294,54 @@ extern "C" int cmk_min_bmm_f32(const float* A, const float* B, float* values, lo
     if (int e = hip_status(hipGetLastError(), "cmk_min_bmm_f32 fold launch")) return e;
   }
   return CMK_OK;
+}
+
+extern "C" int cmk_min_bmm_f32(const float* A, const float* B, float* values, long long* indices,
+                               const cmk_gemm_desc* d, int dim, int distance, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+  return min_bmm_enqueue(A, B, values, indices, d, dim, distance, workspace, workspace_bytes, stream);
+}
+
+// Scratch of the allocation-free entry point: one array per GPU, created with
+// the code object and kept until the process ends.  In host code this name is
+// only a handle for hipGetSymbolAddress; kernels and copies get the device
+// address that call returns.
+static __device__ __align__(256) unsigned char scratch[CMK_STATIC_SCRATCH_BYTES];
+
+namespace cmk {
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_scratch(void** out) {
+  int dev = -1;
+  if (int e = hip_status(hipGetDevice(&dev), "cmk_min_bmm_f32_static: hipGetDevice")) return e;
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(CMK_ERR_UNSUPPORTED, "cmk_min_bmm_f32_static: device ordinal %d beyond %d", dev, kMaxDevices - 1);
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (int e = hip_status(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)),
+                           "cmk_min_bmm_f32_static: hipGetSymbolAddress"))
+      return e;
+    if (!p) return fail(CMK_ERR_UNSUPPORTED, "cmk_min_bmm_f32_static: no address for the scratch array");
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return CMK_OK;
+}
+}  // namespace cmk
+
+extern "C" int cmk_min_bmm_f32_static(const float* A, const float* B, float* values, long long* indices,
+                                      const cmk_gemm_desc* d, int dim, int distance, void* stream) {
+  if (int e = check_desc(d)) return e;
+  if (dim != 1 && dim != 2) return fail(CMK_ERR_INVALID_ARG, "cmk_min_bmm_f32_static: dim must be 1 or 2");
+  const size_t need = cmk_workspace_bytes(CMK_OP_MIN_BMM, d->L, d->M, d->N, d->K, dim);
+  if (need > (size_t)CMK_STATIC_SCRATCH_BYTES)
+    return fail(CMK_ERR_WORKSPACE,
+                "cmk_min_bmm_f32_static: this problem needs %zu bytes of scratch, the static array holds %zu; "
+                "use cmk_min_bmm_f32 with a workspace", need, (size_t)CMK_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (need > 0)
+    if (int e = static_scratch(&ws)) return e;
+  return min_bmm_enqueue(A, B, values, indices, d, dim, distance, ws, need, stream);
 }

@@ -113,6 +113,24 @@ int cmk_min_bmm_f32(const float* A, const float* B,
                     void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * cmk_min_bmm_f32 for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * same arguments without the workspace, same results.  The partial results of
+ * a split reduction go to a static device array of CMK_STATIC_SCRATCH_BYTES
+ * that each GPU holds from library load until the process ends; the call
+ * allocates and frees nothing.  Problems whose cmk_workspace_bytes() exceeds
+ * that size are refused with CMK_ERR_WORKSPACE.  All calls on one GPU share
+ * the array: calls that may overlap on one GPU (different streams) race and
+ * must be serialised by the caller.  No counterpart in the reference, which
+ * allocates through PyTorch at every call (minbmm.py:116-122).
+ */
+#define CMK_STATIC_SCRATCH_BYTES (4u << 20)
+int cmk_min_bmm_f32_static(const float* A, const float* B,
+                           float* values, long long* indices,
+                           const cmk_gemm_desc* d, int dim, int distance,
+                           void* stream);
+
+/*
  * Fused top-k (largest, sorted descending, 0 < k <= 128) of C = A@B (or of
  * the accumulated distance CMK_DIST_*; still the largest k) along `dim` of
  * C[L][M][N]: dim == 2 gives [L][M][k], dim == 1 gives [L][N][k].
