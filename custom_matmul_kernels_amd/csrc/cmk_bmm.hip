@@ -282,8 +282,6 @@ extern "C" int cmk_mbmm_f32(const float* A, const float* B, float* C, const uint
                             const uint8_t* thread_mask, const uint8_t* element_mask,
                             int share_mask, const cmk_gemm_desc* d, void* stream) {
   if (int e = check_desc(d)) return e;
-  if (d->transA || d->transB)
-    return fail(CMK_ERR_UNSUPPORTED, "cmk_mbmm_f32: only the \"nn\" layout is implemented");
   if (d->L == 0 || d->M == 0 || d->N == 0) return CMK_OK;
   if (!C || (d->K > 0 && (!A || !B)) || !block_mask || !thread_mask || !element_mask)
     return fail(CMK_ERR_INVALID_ARG, "cmk_mbmm_f32: null pointer");
@@ -293,5 +291,5 @@ extern "C" int cmk_mbmm_f32(const float* A, const float* B, float* C, const uint
   a.thread_mask = thread_mask;
   a.element_mask = element_mask;
   a.mask_batched = share_mask ? 0 : 1;
-  return hip_status(launch_bmm<true>(a, 0, 0, (hipStream_t)stream), "cmk_mbmm_f32 launch");
+  return hip_status(launch_bmm<true>(a, d->transA, d->transB, (hipStream_t)stream), "cmk_mbmm_f32 launch");
 }

@@ -97,8 +97,20 @@ __device__ __forceinline__ int masks_ge(const uint32_t (&raw)[NR], uint32_t t,
 // lanes and writes them as entries to out[0..128) (LDS owned by this wave).
 // `cand` is kCand entries of wave-private LDS scratch.  `seed` carries the
 // threshold key from one call to the next (0 = none); idx_of(j) is the index of
-// candidate raw[j] of this lane.  Ties at the threshold: earliest (register,
-// lane) position first.  Fewer than 128 real candidates leave empty entries.
+// candidate raw[j] of this lane.  Fewer than 128 real candidates leave empty
+// entries.
+//
+// Ties at the threshold go to the lowest indices, by this invariant: candidates
+// are always taken in the order reg_order(0), reg_order(1), ... (lanes ascending
+// within a register), callers hand over candidates whose indices ascend in that
+// order among equal keys, and the output keeps equal keys in the order they were
+// taken.  With NR == 18 registers 16 and 17 are a running list (the output of an
+// earlier call, over lower indices) and are taken first.
+template <int NR>
+__device__ __forceinline__ constexpr int reg_order(int pos) {
+  return NR == 18 ? (pos < 2 ? 16 + pos : pos - 2) : pos;
+}
+
 template <int NR, class IdxOf>
 __device__ __forceinline__ void select128(const uint32_t (&raw)[NR], IdxOf&& idx_of,
                                           uint32_t& seed, entry_t* cand, entry_t* out) {
@@ -132,12 +144,14 @@ __device__ __forceinline__ void select128(const uint32_t (&raw)[NR], IdxOf&& idx
 
   if (c_lo <= kCand) {
     if (counted != lo) masks_ge(raw, lo, m);
-    // every candidate with a key >= lo goes to the candidate list, in (register,
-    // lane) order, as (raw, ~index); there are at least 128 and at most 256
+    // every candidate with a key >= lo goes to the candidate list, registers in
+    // reg_order and lanes ascending, as (raw, ~index); there are at least 128 and
+    // at most 256
     int base[NR];
-    base[0] = 0;
+    base[reg_order<NR>(0)] = 0;
 #pragma unroll
-    for (int j = 1; j < NR; ++j) base[j] = base[j - 1] + __popcll(m[j - 1]);
+    for (int p = 1; p < NR; ++p)
+      base[reg_order<NR>(p)] = base[reg_order<NR>(p - 1)] + __popcll(m[reg_order<NR>(p - 1)]);
 #pragma unroll
     for (int j = 0; j < NR; ++j) {
       const int pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m[j] >> 32),
@@ -220,10 +234,13 @@ __device__ __forceinline__ void select128(const uint32_t (&raw)[NR], IdxOf&& idx
     }
   } else {
     // more than 256 candidates share the key lo (hi == lo + 1): take every
-    // candidate above lo, then the first ones equal to lo
+    // candidate above lo, then the first ones equal to lo.  `out` may be the list
+    // that registers 16 and 17 were read from; it is only written after every
+    // lane holds its candidates in registers, which the ballots below imply.
     int base = 0;
 #pragma unroll
-    for (int j = 0; j < NR; ++j) {
+    for (int p = 0; p < NR; ++p) {
+      const int j = reg_order<NR>(p);
       const uint32_t key = raw2key(raw[j]);
       const bool g = key > lo;
       const unsigned long long mm = __ballot(g);
@@ -231,11 +248,12 @@ __device__ __forceinline__ void select128(const uint32_t (&raw)[NR], IdxOf&& idx
       base += __popcll(mm);
     }
 #pragma unroll
-    for (int j = 0; j < NR; ++j) {
+    for (int p = 0; p < NR; ++p) {
+      const int j = reg_order<NR>(p);
       const bool tie = raw2key(raw[j]) == lo;
       const unsigned long long mm = __ballot(tie);
-      const int p = base + prefix_in(mm);
-      if (tie && p < kTop) out[p] = lo ? pack_entry(lo, idx_of(j)) : 0ull;
+      const int q = base + prefix_in(mm);
+      if (tie && q < kTop) out[q] = lo ? pack_entry(lo, idx_of(j)) : 0ull;
       base += __popcll(mm);
     }
   }

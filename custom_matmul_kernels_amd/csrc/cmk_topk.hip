@@ -191,7 +191,9 @@ extern "C" int cmk_topk_bmm_f32(const float* A, const float* B, float* values, l
   const long long machine = 2ll * compute_units();
   const dim3 grid((unsigned)(padded < machine ? padded : machine)), block(kTopkThreads);
   hipStream_t st = (hipStream_t)stream;
-  const bool multi = a.splits > 1 || a.xtiles > kChunkTiles;
+  // an empty reduced axis takes the multi-chunk instance, whose lists start out
+  // empty: every slot of the result is then -inf / -1
+  const bool multi = a.splits > 1 || a.xtiles > kChunkTiles || a.xtiles == 0;
   if (distance == CMK_DIST_INNER) launch_topk_kernel<kInner>(xk, yk, multi, grid, block, st, a);
   else launch_topk_dist(distance, xk, yk, multi, grid, block, st, a);
   if (int e = hip_status(hipGetLastError(), "cmk_topk_bmm_f32 launch")) return e;

@@ -15,7 +15,12 @@ class MBMMCUDA:
     file that does not exist, mbmm.py:18); its intended behaviour is taken from
     kernels/mbmm.cu:208-374: C = (A@B) * element_mask where the tile's
     block_mask and the 8x8 micro-tile's thread_mask are non-zero, 0 elsewhere.
-    As in the reference only mode "nn" is implemented.
+    All four modes run (the reference's `_call_tt/_tn/_nt` raise
+    NotImplementedError, mbmm.py:100-107, and its kernels for them are empty):
+    `mode` says how A and B are stored, as the reference documents it
+    (mbmm.py:163-170): "tn" takes A as [l, k, m] and computes A.T @ B, "nt" takes B
+    as [l, n, k] and computes A @ B.T, "tt" both.  Operands whose strides already
+    describe one of the two layouts are consumed in place.
     """
 
     def __init__(self, patch_m=4, patch_n=4, share_mask=False):
@@ -25,7 +30,8 @@ class MBMMCUDA:
         self.share_mask = share_mask
         self._lib = _lib.load()
 
-    def _call_nn(self, A, B, block_mask, thread_mask, element_mask):
+    def _call(self, A, B, block_mask, thread_mask, element_mask):
+        """A [l, m, k] and B [l, k, n] as logical views with any strides."""
         _common.check_operands(A, B)
         l, m, k = A.shape
         n = B.shape[2]
@@ -53,14 +59,17 @@ class MBMMCUDA:
                     1 if self.share_mask else 0, desc, _common.stream_ptr(A.device)))
         return C
 
+    def _call_nn(self, A, B, block_mask, thread_mask, element_mask):
+        return self._call(A, B, block_mask, thread_mask, element_mask)
+
     def _call_tt(self, A, B, block_mask, thread_mask, element_mask):
-        raise NotImplementedError
+        return self._call(A.transpose(1, 2), B.transpose(1, 2), block_mask, thread_mask, element_mask)
 
     def _call_tn(self, A, B, block_mask, thread_mask, element_mask):
-        raise NotImplementedError
+        return self._call(A.transpose(1, 2), B, block_mask, thread_mask, element_mask)
 
     def _call_nt(self, A, B, block_mask, thread_mask, element_mask):
-        raise NotImplementedError
+        return self._call(A, B.transpose(1, 2), block_mask, thread_mask, element_mask)
 
     def __call__(self, A, B, block_mask, thread_mask, element_mask, mode="nn"):
         """
@@ -69,12 +78,11 @@ class MBMMCUDA:
         element_mask: uint8 [m, n] (share_mask) or [l, m, n]
         block_mask:   uint8 [ceil(m/128), ceil(n/128)] or with leading l
         thread_mask:  uint8 [ceil(m/8), ceil(n/8)] or with leading l
-        mode: {"nn", "tn", "nt", "tt"}; only "nn" is implemented
+        mode: {"nn", "tn", "nt", "tt"}: "t" for A means it is given as [l, k, m],
+              "t" for B that it is given as [l, n, k]
         returns C: float32 [m, n] or [l, m, n]
         """
         assert len(A.shape) == len(B.shape)
-        A = A.contiguous()
-        B = B.contiguous()
         two_dimensional = A.dim() == 2 and B.dim() == 2
         if two_dimensional:
             A2, B2 = A[None], B[None]

@@ -78,9 +78,14 @@ int cmk_bmm_f32(const float* A, const float* B, float* C,
  * Tiles whose block_mask is 0 are not computed (only zeros are written).
  * Masks are uint8: block_mask [Lm][ceil(M/128)][ceil(N/128)], thread_mask
  * [Lm][ceil(M/8)][ceil(N/8)], element_mask [Lm][M][N] with Lm = 1 when
- * share_mask != 0 and Lm = L otherwise.  Only transA == transB == 0 is
- * accepted, as in the reference.  Replaces the launch of mbmm_nn
- * (reference mbmm.py:84-97, kernels/mbmm.cu:208-374).
+ * share_mask != 0 and Lm = L otherwise.  All four operand layouts are
+ * accepted (the reference implements "nn" only; its mbmm_tn / mbmm_nt /
+ * mbmm_tt are empty).  The element mask is a 0/1 multiplier, as in the
+ * reference (kernels/mbmm.cu:127-128): a non-finite product under a zero
+ * element-mask byte gives NaN, not 0; block- and thread-masked positions are
+ * exact zeros whatever the operands hold.  Replaces the launch of mbmm_nn
+ * (reference mbmm.py:84-97, kernels/mbmm.cu:208-374) and stands in for
+ * mbmm_tn, mbmm_nt, mbmm_tt (kernels/mbmm.cu:184-206, 376-385).
  */
 int cmk_mbmm_f32(const float* A, const float* B, float* C,
                  const uint8_t* block_mask, const uint8_t* thread_mask,

@@ -75,8 +75,9 @@ def test_argument_errors_return_codes_without_launching(lib):
     assert lib.cmk_bmm_f32(fake, fake, fake, _desc(lda=4), None) == _lib.ERR_INVALID_ARG
     assert lib.cmk_bmm_f32(fake, fake, fake, _desc(tA=2), None) == _lib.ERR_INVALID_ARG
     assert lib.cmk_bmm_f32(None, fake, fake, _desc(), None) == _lib.ERR_INVALID_ARG
-    assert lib.cmk_mbmm_f32(fake, fake, fake, fake, fake, fake, 0, _desc(tA=1, lda=8), None) \
-        == _lib.ERR_UNSUPPORTED
+    assert lib.cmk_mbmm_f32(fake, fake, fake, fake, fake, fake, 0, _desc(tA=1, M=16, lda=8), None) \
+        == _lib.ERR_INVALID_ARG            # "t" layout of A: lda must cover m
+    assert lib.cmk_mbmm_f32(fake, fake, fake, None, fake, fake, 0, _desc(), None) == _lib.ERR_INVALID_ARG
     assert lib.cmk_min_bmm_f32(fake, fake, fake, fake, _desc(), 3, 0, None, 0, None) \
         == _lib.ERR_INVALID_ARG
     assert lib.cmk_min_bmm_f32(fake, fake, fake, fake, _desc(), 2, 7, None, 0, None) \

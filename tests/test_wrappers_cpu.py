@@ -86,9 +86,16 @@ def test_shape_and_dtype_checks_fire_before_any_launch():
         MBMMCUDA(share_mask=1)
     mb = MBMMCUDA()
     u8 = torch.uint8
-    with pytest.raises(NotImplementedError):
+    # every mode is dispatched ("tn": A is [l, k, m]); CPU tensors are refused after the shape checks
+    with pytest.raises(AssertionError):
         mb(torch.zeros(1, 8, 8), torch.zeros(1, 8, 8), torch.zeros(1, 1, 1, dtype=u8),
            torch.zeros(1, 1, 1, dtype=u8), torch.zeros(1, 8, 8, dtype=u8), mode="tn")
+    with pytest.raises(AssertionError):
+        mb(torch.zeros(1, 5, 8), torch.zeros(1, 8, 8), torch.zeros(1, 1, 1, dtype=u8),
+           torch.zeros(1, 1, 1, dtype=u8), torch.zeros(1, 8, 8, dtype=u8), mode="tn")   # k: 5 vs 8
+    with pytest.raises(KeyError):
+        mb(torch.zeros(1, 8, 8), torch.zeros(1, 8, 8), torch.zeros(1, 1, 1, dtype=u8),
+           torch.zeros(1, 1, 1, dtype=u8), torch.zeros(1, 8, 8, dtype=u8), mode="xx")
 
 
 def test_derive_masks_rejects_host_tensors_and_other_dtypes():
