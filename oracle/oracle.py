@@ -211,8 +211,6 @@ def check_values(got, want, K, what="values"):
 def gather_products(A, B, dim, indices):
     """C[l, y, indices[l, y, ...]] recomputed in float64 without forming C.
     A [l,m,k], B [l,k,n] CPU tensors; indices [l, kept] or [l, kept, q]."""
-    A = A.double()
-    B = B.double()
     if dim == 1:
         A, B = B.transpose(1, 2), A.transpose(1, 2)
     idx = indices if indices.dim() == 3 else indices[..., None]
@@ -220,10 +218,11 @@ def gather_products(A, B, dim, indices):
     out = torch.empty(l, kept, q, dtype=torch.float64)
     safe = idx.clamp(min=0)
     step = max(1, (1 << 24) // max(1, q * A.shape[2]))
+    bt = B.transpose(1, 2)                                       # [l, X, K]
     for r0 in range(0, kept, step):
-        a = A[:, r0:r0 + step]                                   # [l, r, K]
-        bt = B.transpose(1, 2)                                   # [l, X, K]
-        sel = torch.stack([bt[b][safe[b, r0:r0 + step]] for b in range(l)])  # [l, r, q, K]
+        a = A[:, r0:r0 + step].double()                          # [l, r, K]
+        # only the gathered columns are widened, never the whole operand
+        sel = torch.stack([bt[b][safe[b, r0:r0 + step]] for b in range(l)]).double()  # [l, r, q, K]
         out[:, r0:r0 + step] = (a[:, :, None, :] * sel).sum(-1)
     return out if indices.dim() == 3 else out[..., 0]
 
