@@ -157,10 +157,11 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
 }
 
 // Folds the per-split partial results in ascending split (= ascending index)
-// order.  The partials of eight splits are requested together, so that the
-// kernel waits for memory once per eight splits instead of once per split; 64
-// threads per work-group spread a small problem over more CUs.
+// order.  The partials of up to sixteen splits are requested together, so that
+// the kernel waits for memory once (the usual plans have at most sixteen splits);
+// 64 threads per work-group spread a small problem over more CUs.
 constexpr int kFoldThreads = 64;
+constexpr int kFoldBatch = 16;
 __global__ __launch_bounds__(kFoldThreads) void min_fold_kernel(const float* part_val, const int* part_idx,
                                                                 float* values, long long* indices,
                                                                 long long rows, int splits) {
@@ -168,17 +169,17 @@ __global__ __launch_bounds__(kFoldThreads) void min_fold_kernel(const float* par
   if (i >= rows) return;
   float v = INFINITY;
   int idx = part_idx[i];
-  for (int s0 = 0; s0 < splits; s0 += 8) {
-    float pv[8];
-    int pi[8];
+  for (int s0 = 0; s0 < splits; s0 += kFoldBatch) {
+    float pv[kFoldBatch];
+    int pi[kFoldBatch];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < kFoldBatch; ++j) {
       const int s = s0 + j < splits ? s0 + j : splits - 1;   // clamped: repeats fold to nothing
       pv[j] = part_val[(long long)s * rows + i];
       pi[j] = part_idx[(long long)s * rows + i];
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+    for (int j = 0; j < kFoldBatch; ++j)
       if (pv[j] < v) { v = pv[j]; idx = pi[j]; }
   }
   values[i] = v;
