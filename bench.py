@@ -44,9 +44,18 @@ PEAK_VALU_TOPS = 39.3           # 256 CUs x 64 lanes x 2.4 GHz: one fp32 vector 
 # traffic = (2 * FETCH_SIZE + WRITE_SIZE) * 1024.  The counters cannot be read
 # from inside this process; each figure names the summary it was taken from.
 MEASURED_TRAFFIC = {
-    "min_bmm_large": ((2 * 2.15038e6 + 2048) * 1024, "profiles/min_kernel_min_bmm_large.txt"),
-    "topk_bmm": ((2 * 882558 + 1.71006e6) * 1024, "profiles/topk_kernel_topk_bmm.txt"),
-    "derive_masks_4GiB": ((2 * 2.09726e6 + 66564.6) * 1024, "profiles/derive_masks_kernel_4GiB.txt"),
+    "min_bmm_large": ((2 * 2.12432e6 + 2048) * 1024, "profiles/min_kernel_min_bmm_large.txt"),
+    "min_bmm_small": ((2 * 4711.57 + 512) * 1024, "profiles/min_kernel_min_bmm_small.txt"),
+    "bmm": ((2 * 65926.9 + 524291) * 1024, "profiles/bmm_kernel_bmm.txt"),
+    "mbmm": ((2 * 48340 + 524291) * 1024, "profiles/bmm_kernel_mbmm.txt"),
+    "ref_mbmm_tril_1024": ((2 * 70793.2 + 524290) * 1024, "profiles/bmm_kernel_ref_mbmm_tril_1024.txt"),
+    "topk_bmm": ((2 * 882178 + 1.71004e6) * 1024, "profiles/topk_kernel_topk_bmm.txt"),
+    "topk_bmm_k64": ((2 * 191286 + 1.70621e6) * 1024, "profiles/topk_kernel_topk_bmm_k64.txt"),
+    "topk_bmm_nt": ((2 * 232602 + 499713) * 1024, "profiles/topk_kernel_topk_bmm_nt.txt"),
+    "topk_bmm_multi": ((2 * 402063 + 378880) * 1024, "profiles/topk_kernel_topk_bmm_multi.txt"),
+    "topk_bmm_l2": ((2 * 13468.7 + 108959) * 1024, "profiles/topk_kernel_topk_bmm_l2.txt"),
+    "ref_topk_bmm_32768_dim1": ((2 * 56118.1 + 77626) * 1024, "profiles/topk_kernel_ref_topk_bmm_32768_dim1.txt"),
+    "derive_masks_4GiB": ((2 * 2.09725e6 + 66564) * 1024, "profiles/derive_masks_kernel_4GiB.txt"),
 }
 
 SEED = 0
@@ -125,12 +134,16 @@ def make_workloads(torch, cmk, O, dev):
             w["config"] = config
         W[name] = w
 
-    def topk_wl(name, L, M, N, K, dim=2, cpu_rows=None, config=None):
-        op = cmk.TopkBMMCUDA()
+    def topk_wl(name, L, M, N, K, dim=2, cpu_rows=None, config=None, b_transposed=False, distance="inner"):
+        op = cmk.TopkBMMCUDA(distance=distance)
+        inner = distance == "inner"
 
         def make():
             A, B = randn_pair(L, M, N, K)
-            return (A, B), to_dev(A, B)
+            Ad, Bd = to_dev(A, B)
+            if b_transposed:                         # B stored [n, k]: the "nt" layout of the reference
+                Bd = Bd.transpose(1, 2).contiguous().transpose(1, 2)
+            return (A, B), (Ad, Bd)
 
         def parity(cpu_args, dev_args, out):
             A, B = cpu_args
@@ -141,13 +154,23 @@ def make_workloads(torch, cmk, O, dev):
                 As, Bs = A[:, rows], B
             else:
                 As, Bs = A, B[:, :, rows]
+            if not inner:
+                cv, ci = O.c_topk_bmm(As.numpy(), Bs.numpy(), 128, dim, 1 if distance == "l2" else 2)
+                assert torch.equal(v[:, rows].cpu(), torch.from_numpy(cv)), "values differ from the C oracle"
+                return "%d of %d output rows: values bit-equal to the C oracle's %s accumulation and selection" % (
+                    len(rows), kept, distance)
             mism = O.check_topk(v[:, rows].cpu(), i[:, rows].cpu(), As, Bs, 128, dim)
             return "%d of %d output rows per batch against torch.bmm(A,B).topk(128) on the CPU (values, order, " \
                    "value-at-index, uniqueness); %d index differences, all between products closer than the " \
                    "tolerance" % (len(rows), kept, mism)
 
-        w = dict(make=make, run=lambda A, B: op(A, B, k=128, dim=dim), flop=2.0 * L * M * N * K, parity=parity,
-                 desc="topk_bmm fp32 A[%d,%d,%d] @ B[%d,%d,%d], k=128 over dim=%d" % (L, M, K, L, K, N, dim))
+        per = 2.0 if inner else (3.0 if distance == "l2" else 2.0)
+        w = dict(make=make, run=lambda A, B: op(A, B, k=128, dim=dim), flop=per * L * M * N * K, parity=parity,
+                 desc="topk_bmm%s fp32 A[%d,%d,%d] @ B[%d,%d,%d]%s, k=128 over dim=%d" % (
+                     "" if inner else " distance=" + distance, L, M, K, L, K, N,
+                     " (B stored [n,k])" if b_transposed else "", dim))
+        if not inner:
+            w["valu_ops"] = 2.0 * L * M * N * K
         if cpu_rows:
             w.update(cpu=lambda A, B, r0: torch.bmm(A[:, r0:r0 + cpu_rows], B).topk(128, dim=-1), cpu_rows=cpu_rows,
                      rows=M, cpu_flop_per_row=2.0 * L * N * K, cpu_expr="torch.bmm(A,B).topk(128,-1)")
@@ -272,6 +295,10 @@ def make_workloads(torch, cmk, O, dev):
     topk_wl("ref_topk_bmm_2e20_k256_dim1", 1, 1048576, 1024, 256, dim=1)   # imgs/topk_bmm_A[1,N,256] ..._loglog.png
     topk_wl("ref_topk_bmm_2e20_k1024_dim1", 1, 1048576, 1024, 1024, dim=1)  # imgs/topk_bmm_A[1,N,1024] ..._loglog.png
     topk_wl("topk_bmm_k64", 1, 1048576, 1024, 64)              # the fused top-k at K = 64, dim=-1
+    # other code paths of the top-k kernel: B stored [n,k], a reduced axis of several chunks, a vector-unit distance
+    topk_wl("topk_bmm_nt", 1, 262144, 1024, 256, b_transposed=True)
+    topk_wl("topk_bmm_multi", 1, 16384, 16384, 256)
+    topk_wl("topk_bmm_l2", 1, 65536, 1024, 64, distance="l2")
     return W
 
 
