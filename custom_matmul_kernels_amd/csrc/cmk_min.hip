@@ -43,14 +43,17 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
   // `ygroup` y strips x `splits` ranges of X: the strips of Y they re-read for
   // every tile stay in that XCD's L2, and each X tile is fetched once for the
   // `ygroup` work-groups that walk the same range.
+  // Every id is a real work slot (a padded last group would push whole XCDs into
+  // a second round): the last group simply has fewer strips.
   const int logical = xcd_logical_id(blockIdx.x, a.total);
   if (logical < 0) return;
   const int gsz = a.ygroup * a.splits;
   const int group = logical / gsz;
+  const int ybase = group * a.ygroup;
+  const int yg = min(a.ygroup, a.L * a.ystrips - ybase);   // strips of this group
   const int within = logical - group * gsz;
-  const int split = within / a.ygroup;
-  const int yflat = group * a.ygroup + within % a.ygroup;
-  if (yflat >= a.L * a.ystrips) return;
+  const int split = within / yg;
+  const int yflat = ybase + within % yg;
   const int b = yflat / a.ystrips;
   const int ystrip = yflat - b * a.ystrips;
   const int y0 = ystrip * C::TY;
@@ -189,9 +192,11 @@ __global__ __launch_bounds__(kFoldThreads) void min_fold_kernel(const float* par
 // How the work is cut.  Splitting the reduced axis gives more work-groups than
 // the kept axis alone has strips; every candidate split count is priced as
 // (rounds the machine needs for all work-groups, two per CU) x (slabs one
-// work-group multiplies + a fixed cost for filling the pipeline and folding) and
-// the cheapest is taken.  When X is too large to stay in an XCD's L2 at least
-// four splits are used, so that fewer distinct Y strips are live per XCD.
+// work-group multiplies + what a work-group costs besides: filling the pipeline
+// and the reduction across lanes and waves, measured at 2.2 us against 3.4 us per
+// slab) + the fold launch when there is a split (about one slab), in quarter
+// slabs, and the cheapest is taken.  When X is too large to stay in an XCD's L2
+// at least four splits are used, so that fewer distinct Y strips are live per XCD.
 static void plan_min(int L, int Xext, int Yext, int K, int* ystrips, int* xtiles, int* splits,
                      int* tiles_per_split, int* ygroup) {
   *ystrips = ceil_div(Yext, 128);
@@ -206,10 +211,9 @@ static void plan_min(int L, int Xext, int Yext, int K, int* ystrips, int* xtiles
   for (int want = big_x ? 4 : 1; want <= most; ++want) {
     const int tps = ceil_div(*xtiles, want);
     const int s = ceil_div(*xtiles, tps);
-    const int yg = 64 / s > 0 ? 64 / s : 1;
-    const long long total = ((strips + yg - 1) / yg) * yg * s;
+    const long long total = strips * s;
     const long long rounds = (total + slots - 1) / slots;
-    const long long cost = rounds * (tps * slabs + 6);
+    const long long cost = rounds * (4 * tps * slabs + 3) + (s > 1 ? 4 : 0);
     if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_tps = tps; }
   }
   *tiles_per_split = best_tps;
@@ -268,8 +272,7 @@ static int min_bmm_enqueue(const float* A, const float* B, float* values, long l
     a.part_val = static_cast<float*>(workspace);
     a.part_idx = reinterpret_cast<int*>(a.part_val + (size_t)a.splits * d->L * Yext);
   }
-  const long long ytot = (long long)d->L * a.ystrips;
-  const long long total = ((ytot + a.ygroup - 1) / a.ygroup) * a.ygroup * a.splits;
+  const long long total = (long long)d->L * a.ystrips * a.splits;
   if (int e = check_grid(total)) return e;
   a.total = (int)total;
   const dim3 grid((unsigned)(((total + 7) / 8) * 8)), block(kThreads);
