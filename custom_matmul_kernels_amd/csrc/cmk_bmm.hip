@@ -27,9 +27,12 @@ struct BmmArgs {
 constexpr int kMaskRows = 128;    // element-mask tile staged in LDS: rows ...
 constexpr int kMaskPitch = 144;   // ... of 128 bytes, 16-byte aligned, skewed over the banks
 
-template <int XK, int YK, bool MASKED>
+// B = 32x32 blocks per wave and axis: 2 gives the 128x128 tile, 1 a 64x64 tile
+// for products with too few 128x128 tiles to occupy the chip (dense only).
+template <int XK, int YK, bool MASKED, int B = 2>
 __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
-  using C = Core<XK, YK, 2, 2, 2, 2>;
+  using C = Core<XK, YK, 2, 2, B, B>;
+  static_assert(B == 2 || !MASKED, "the masks are laid out for 128x128 tiles");
   __shared__ __attribute__((aligned(16))) float lds[C::ldsFloats];
 
   // A work-group owns `run` consecutive tiles along m of one 128-wide column
@@ -90,7 +93,7 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
   for (int ti = 0; ti < ntiles; ++ti) {
     // the dense product starts its accumulators from a literal zero; for the
     // masked one that form measured slower (191 vs 165 us at the benchmark shape)
-    f32x16 acc[2][2];
+    f32x16 acc[B][B];
     if constexpr (MASKED) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
@@ -136,9 +139,9 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
     // C is written once and not read again here: non-temporal stores keep it from
     // displacing the operands in L2 (measured: 4 % on the dense product)
     const int wv = __builtin_amdgcn_readfirstlane(wave);
-    const int mw = (tile_m0 + ti) * C::TX + (wv % 2) * 64;
-    const int nw = n0 + (wv / 2) * 64;
-    if (mw + 64 <= a.M && nw + 64 <= a.N && (long long)a.N * 68 * 4 < (1ll << 31)) {
+    const int mw = (tile_m0 + ti) * C::TX + (wv % 2) * 32 * B;
+    const int nw = n0 + (wv / 2) * 32 * B;
+    if (mw + 32 * B <= a.M && nw + 32 * B <= a.N && (long long)a.N * 68 * 4 < (1ll << 31)) {
       // interior: row addresses are scalar, the lane part is one 32-bit offset
       typedef float __attribute__((address_space(1))) * gfp;
       typedef const uint8_t __attribute__((address_space(1))) * gbp;
@@ -146,12 +149,12 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
       const unsigned voff = static_cast<unsigned>((4 * half * a.N + l32) * 4);
       if constexpr (!MASKED) {
 #pragma unroll
-        for (int bx = 0; bx < 2; ++bx)
+        for (int bx = 0; bx < B; ++bx)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             char* rp = base + (long long)(bx * 32 + 8 * (r >> 2) + (r & 3)) * a.N * 4;
 #pragma unroll
-            for (int by = 0; by < 2; ++by) __builtin_nontemporal_store(acc[bx][by][r], (gfp)(rp + voff + by * 128));
+            for (int by = 0; by < B; ++by) __builtin_nontemporal_store(acc[bx][by][r], (gfp)(rp + voff + by * 128));
           }
       } else if (staged) {
         // masks come from LDS: byte reads there cost no vector-memory instructions
@@ -209,9 +212,9 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
       }
     } else {
 #pragma unroll
-      for (int bx = 0; bx < 2; ++bx) {
+      for (int bx = 0; bx < B; ++bx) {
 #pragma unroll
-        for (int by = 0; by < 2; ++by) {
+        for (int by = 0; by < B; ++by) {
           const int n = nw + by * 32 + l32;
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
@@ -234,26 +237,26 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
   }
 }
 
-template <bool MASKED>
+template <bool MASKED, int B = 2>
 static hipError_t launch_bmm(const BmmArgs& a, int transA, int transB, hipStream_t st) {
   const int total = a.L * ((a.tiles_m + a.run - 1) / a.run) * a.tiles_n;
   const dim3 grid(((total + 7) / 8) * 8), block(kThreads);
   // A "n" is k-contiguous (KC), A "t" is m-contiguous (RC);
   // B "n" is n-contiguous (RC), B "t" is k-contiguous (KC).
-  if (!transA && !transB) hipLaunchKernelGGL((bmm_kernel<KC, RC, MASKED>), grid, block, 0, st, a);
-  else if (!transA && transB) hipLaunchKernelGGL((bmm_kernel<KC, KC, MASKED>), grid, block, 0, st, a);
-  else if (transA && !transB) hipLaunchKernelGGL((bmm_kernel<RC, RC, MASKED>), grid, block, 0, st, a);
-  else hipLaunchKernelGGL((bmm_kernel<RC, KC, MASKED>), grid, block, 0, st, a);
+  if (!transA && !transB) hipLaunchKernelGGL((bmm_kernel<KC, RC, MASKED, B>), grid, block, 0, st, a);
+  else if (!transA && transB) hipLaunchKernelGGL((bmm_kernel<KC, KC, MASKED, B>), grid, block, 0, st, a);
+  else if (transA && !transB) hipLaunchKernelGGL((bmm_kernel<RC, RC, MASKED, B>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((bmm_kernel<RC, KC, MASKED, B>), grid, block, 0, st, a);
   return hipGetLastError();
 }
 
-static BmmArgs make_args(const float* A, const float* B, float* C, const cmk_gemm_desc* d) {
+static BmmArgs make_args(const float* A, const float* B, float* C, const cmk_gemm_desc* d, int tile = 128) {
   BmmArgs a{};
   a.A = A; a.B = B; a.C = C;
   a.lda = d->lda; a.ldb = d->ldb; a.strideA = d->strideA; a.strideB = d->strideB;
   a.L = d->L; a.M = d->M; a.N = d->N; a.K = d->K;
-  a.tiles_m = (d->M + 127) / 128;
-  a.tiles_n = (d->N + 127) / 128;
+  a.tiles_m = (d->M + tile - 1) / tile;
+  a.tiles_n = (d->N + tile - 1) / tile;
   a.run = 1;
   a.vecA = vec_ok(A, d->lda, d->strideA);
   a.vecB = vec_ok(B, d->ldb, d->strideB);
@@ -271,8 +274,15 @@ extern "C" int cmk_bmm_f32(const float* A, const float* B, float* C, const cmk_g
   if (!C || (d->K > 0 && (!A || !B))) return fail(CMK_ERR_INVALID_ARG, "cmk_bmm_f32: null pointer");
   if (int e = check_grid((long long)d->L * ((d->M + 127) / 128) * ((d->N + 127) / 128))) return e;
   BmmArgs a = make_args(A, B, C, d);
-  // longer runs amortise the pipeline fill; keep at least ~4 work-groups per CU
   const long long tiles = (long long)d->L * a.tiles_m * a.tiles_n;
+  if (tiles < 3 * compute_units()) {
+    // too few 128x128 tiles for two even rounds of the chip (measured: up to ~600
+    // tiles the smaller tile wins, at 1024 the larger): 64x64 tiles, four times as many
+    a = make_args(A, B, C, d, 64);
+    return hip_status(launch_bmm<false, 1>(a, d->transA, d->transB, (hipStream_t)stream),
+                      "cmk_bmm_f32 launch");
+  }
+  // longer runs amortise the pipeline fill; keep at least ~4 work-groups per CU
   a.run = tiles >= 8192 ? 4 : (tiles >= 4096 ? 2 : 1);
   return hip_status(launch_bmm<false>(a, d->transA, d->transB, (hipStream_t)stream),
                     "cmk_bmm_f32 launch");

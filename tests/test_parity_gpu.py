@@ -29,8 +29,11 @@ def say(*a):
 
 
 # ---------------------------------------------------------------- bmm --------
+# the last three have enough 128x128 tiles for the large-tile kernel (ragged edges included),
+# the others take the 64x64-tile kernel
 BMM_SHAPES = [(1, 1, 1, 1), (2, 37, 300, 19), (3, 129, 257, 33), (1, 128, 128, 64),
-              (2, 200, 136, 70), (1, 256, 384, 100), (5, 64, 64, 32)]
+              (2, 200, 136, 70), (1, 256, 384, 100), (5, 64, 64, 32),
+              (70, 300, 520, 33), (13, 1000, 1100, 40), (1, 4000, 3100, 24)]
 
 
 @pytest.mark.parametrize("mode", MODES)
