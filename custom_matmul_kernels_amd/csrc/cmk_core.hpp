@@ -181,6 +181,47 @@ __device__ __noinline__ void fetch_edge(const float* p, long long ld, int rows, 
   }
 }
 
+// The same for an operand whose edge tiles can still use direct loads: 16-byte
+// aligned, and the extent that a 16-byte chunk runs along (k for KC, rows for RC)
+// a multiple of 4, so that a chunk lies wholly inside or wholly outside the
+// matrix.  Chunks beyond K are written as zeros; chunks beyond the last row are
+// fetched from the last rows instead (their products belong to output elements
+// that no epilogue uses, and stay finite when the operand is).
+template <int KIND, int T, int KS, int NT>
+__device__ __noinline__ void fetch_edge_direct(const float* p, long long ld, int rows, int K, int r0,
+                                               int k0, float* dst, int tid) {
+  using M = LoadMap<KIND, T, KS, NT>;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+#pragma unroll
+  for (int pp = 0; pp < M::NV; ++pp) {
+    const int q = pp * M::NW + wave;
+    if (!M::kEven && q >= M::NI) continue;
+    int k;
+    long long e;
+    if constexpr (KIND == KC) {
+      constexpr int CPR = KS / 4;
+      const int row = q * (256 / KS) + lane / CPR;
+      const int slot = lane % CPR;
+      const int chunk = ((slot ^ row) & 7) | (slot & ~7);
+      k = k0 + chunk * 4;
+      const int rr = min(r0 + row, rows - 1);
+      e = (long long)rr * ld + k;
+    } else {
+      const int f = q * 256 + lane * 4;
+      k = k0 + f / T;
+      const int rr = min(r0 + f % T, rows - 4);
+      e = (long long)k * ld + rr;
+    }
+    float* piece = dst + q * 256;
+    if (k < K) {
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(p + e), (lds_void_ptr)piece, 16, 0, 0);
+    } else {
+      *reinterpret_cast<f32x4*>(piece + lane * 4) = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+}
+
 // Work-group level tile engine.  WX x WY waves (4, 8 or 16 of them), each wave owns
 // BX x BY blocks of 32x32; KS is the contraction depth of one LDS slab.
 //
@@ -230,8 +271,9 @@ struct Core {
   int xbase, y0, K;
   int xr, yr, half, tid;
   // Interior test of a slab in three scalar subtractions: last first-row (and
-  // last first-k) at which a whole tile still lies inside the matrix; -1 for an
-  // operand that rules out direct loads (unaligned, or offsets beyond 32 bits).
+  // last first-k) at which a whole tile still lies inside the matrix; -2 * tile
+  // size for an operand that rules out direct loads (unaligned, or offsets beyond
+  // 32 bits).
   int xlast, ylast, klast;
   // LDS byte addresses of this lane's fragments in buffer 0, kept in registers
   // for the whole sequence so that a fragment read is (register + immediate):
@@ -281,6 +323,9 @@ struct Core {
           __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + o32),
                                            (lds_void_ptr)(dst + (p * M::NW + wave) * 256), 16, 0, 0);
         }
+    } else if (rlast >= -T && (KIND == KC ? (K & 3) == 0 : (o.rows & 3) == 0)) {
+      // (rlast >= -T: direct loads are legal for this operand and it has at least 4 rows / 1 row)
+      fetch_edge_direct<KIND, T, KS, NT>(o.p, o.ld, o.rows, K, r0, k0, dst, tid);
     } else {
       fetch_edge<KIND, T, KS, NT>(o.p, o.ld, o.rows, K, r0, k0, dst, tid);
     }
@@ -403,8 +448,10 @@ struct Core {
     y0 = __builtin_amdgcn_readfirstlane(y0_);
     K = __builtin_amdgcn_readfirstlane(K_);
     S = max(1, (K + KS - 1) / KS);
-    xlast = (X.vec != 0 && (long long)(TX + KS) * X.ld < (1ll << 29)) ? X.rows - TX : -1;
-    ylast = (Y.vec != 0 && (long long)(TY + KS) * Y.ld < (1ll << 29)) ? Y.rows - TY : -1;
+    // (first row of the last tile that lies wholly inside; negative when there is none;
+    // below -tile size: no direct loads for this operand at all)
+    xlast = (X.vec != 0 && X.rows > 0 && (long long)(TX + KS) * X.ld < (1ll << 29)) ? X.rows - TX : -2 * TX;
+    ylast = (Y.vec != 0 && Y.rows > 0 && (long long)(TY + KS) * Y.ld < (1ll << 29)) ? Y.rows - TY : -2 * TY;
     klast = K - KS;
     nt = __builtin_amdgcn_readfirstlane(ntiles);
     iters = nt * S;
