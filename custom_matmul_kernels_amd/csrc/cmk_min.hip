@@ -86,23 +86,31 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
           for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     }
     core.template tile<DIST, DIST == kInner>(X, Y, lds, acc);
-    // fold this tile into the running minimum; indices ascend within a lane,
-    // so a strict '<' keeps the first occurrence
+    // Fold this tile into the running minimum.  Inside the tile a lane tracks the
+    // position of its minimum as a small code (block * 16 + register: a literal
+    // per compare, no index registers); indices ascend with the code, so a strict
+    // '<' keeps the first occurrence.  The code becomes an index once per tile.
     const int xb = xt * C::TX + wx * 64;
+    float tbest[2];
+    int tcode[2];
     if (xb + 64 <= X.rows) {
+#pragma unroll
+      for (int by = 0; by < 2; ++by) { tbest[by] = acc[0][by][0]; tcode[by] = 0; }
 #pragma unroll
       for (int bx = 0; bx < 2; ++bx)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int x = xb + bx * 32 + acc_row(r, half);
+          if (bx == 0 && r == 0) continue;
 #pragma unroll
           for (int by = 0; by < 2; ++by) {
             const float v = acc[bx][by][r];
-            if (v < best[by]) { best[by] = v; bidx[by] = x; }
+            if (v < tbest[by]) { tbest[by] = v; tcode[by] = bx * 16 + r; }
           }
         }
     } else {
 #pragma unroll
+      for (int by = 0; by < 2; ++by) { tbest[by] = INFINITY; tcode[by] = 0; }
+#pragma unroll
       for (int bx = 0; bx < 2; ++bx)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -110,9 +118,14 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
 #pragma unroll
           for (int by = 0; by < 2; ++by) {
             const float v = acc[bx][by][r];
-            if (x < X.rows && v < best[by]) { best[by] = v; bidx[by] = x; }
+            if (x < X.rows && v < tbest[by]) { tbest[by] = v; tcode[by] = bx * 16 + r; }
           }
         }
+    }
+#pragma unroll
+    for (int by = 0; by < 2; ++by) {
+      const int x = xb + (tcode[by] >> 4) * 32 + acc_row(tcode[by] & 15, half);
+      if (tbest[by] < best[by]) { best[by] = tbest[by]; bidx[by] = x; }
     }
   }
   __syncthreads();  // the operand buffers are reused below
