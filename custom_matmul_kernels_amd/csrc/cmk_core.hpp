@@ -187,8 +187,12 @@ __device__ __noinline__ void fetch_edge(const float* p, long long ld, int rows, 
 // matrix.  Chunks beyond K are written as zeros; chunks beyond the last row are
 // fetched from the last rows instead (their products belong to output elements
 // that no epilogue uses, and stay finite when the operand is).
+// Inlined where registers allow (fetch_edge_direct_call below is the same as a
+// real function): a call waits for the loads before it returns - the calling
+// convention drains the memory counters at function boundaries - so that an edge
+// tile pays the full memory latency once per slab.
 template <int KIND, int T, int KS, int NT>
-__device__ __noinline__ void fetch_edge_direct(const float* p, long long ld, int rows, int K, int r0,
+__device__ __forceinline__ void fetch_edge_direct(const float* p, long long ld, int rows, int K, int r0,
                                                int k0, float* dst, int tid) {
   using M = LoadMap<KIND, T, KS, NT>;
   const int lane = tid & 63;
@@ -220,6 +224,12 @@ __device__ __noinline__ void fetch_edge_direct(const float* p, long long ld, int
       *reinterpret_cast<f32x4*>(piece + lane * 4) = f32x4{0.f, 0.f, 0.f, 0.f};
     }
   }
+}
+
+template <int KIND, int T, int KS, int NT>
+__device__ __noinline__ void fetch_edge_direct_call(const float* p, long long ld, int rows, int K, int r0,
+                                                    int k0, float* dst, int tid) {
+  fetch_edge_direct<KIND, T, KS, NT>(p, ld, rows, K, r0, k0, dst, tid);
 }
 
 // Work-group level tile engine.  WX x WY waves (4, 8 or 16 of them), each wave owns
@@ -325,7 +335,9 @@ struct Core {
         }
     } else if (rlast >= -T && (KIND == KC ? (K & 3) == 0 : (o.rows & 3) == 0)) {
       // (rlast >= -T: direct loads are legal for this operand and it has at least 4 rows / 1 row)
-      fetch_edge_direct<KIND, T, KS, NT>(o.p, o.ld, o.rows, K, r0, k0, dst, tid);
+      // (a kernel that runs without address registers is short of registers altogether)
+      if constexpr (ADDR_REGS) fetch_edge_direct<KIND, T, KS, NT>(o.p, o.ld, o.rows, K, r0, k0, dst, tid);
+      else fetch_edge_direct_call<KIND, T, KS, NT>(o.p, o.ld, o.rows, K, r0, k0, dst, tid);
     } else {
       fetch_edge<KIND, T, KS, NT>(o.p, o.ld, o.rows, K, r0, k0, dst, tid);
     }
