@@ -59,6 +59,34 @@ def _operand(T, want_inner, name):
     return Tc, 0, max(c, 1), r * c
 
 
+# An operand that is not 16-byte aligned (base, leading dimension or batch
+# stride) cannot use the kernels' direct global-to-LDS loads at all and runs
+# about three times slower; between these sizes (elements) a padded copy costs
+# far less than that and does not double a footprint that matters.
+ALIGN_COPY_MIN = 1 << 16
+ALIGN_COPY_MAX = 1 << 28
+
+
+def _aligned(T, trans, ld, stride):
+    """The operand itself when the kernels can fetch it with 16-byte loads (or
+    when a copy is not worth it), otherwise a copy whose rows are padded to a
+    multiple of four elements; the padding is never read."""
+    l, r, c = T.shape
+    if (T.data_ptr() % 16 == 0 and ld % 4 == 0 and stride % 4 == 0) or \
+            not ALIGN_COPY_MIN <= T.numel() <= ALIGN_COPY_MAX:
+        return T, trans, ld, stride
+    inner, outer = (c, r) if trans == 0 else (r, c)
+    ldp = (inner + 3) // 4 * 4
+    buf = torch.empty(l, outer, ldp, dtype=T.dtype, device=T.device)
+    if trans == 0:
+        view = buf[..., :c]
+        view.copy_(T)
+    else:
+        view = buf[..., :r].transpose(1, 2)
+        view.copy_(T)
+    return view, trans, ldp, outer * ldp
+
+
 def make_desc(A, B):
     """Builds the descriptor for C = A @ B with A [l,m,k], B [l,k,n].  The
     returned tensors must stay alive until the launch has been enqueued."""
@@ -69,6 +97,8 @@ def make_desc(A, B):
     if sA < 0 or sB < 0:
         A2, tA, lda, sA = A.contiguous(), 0, max(k, 1), m * k
         B2, tB, ldb, sB = B.contiguous(), 0, max(n, 1), k * n
+    A2, tA, lda, sA = _aligned(A2, tA, lda, sA)
+    B2, tB, ldb, sB = _aligned(B2, tB, ldb, sB)
     # the descriptor's trans flag for A is about [m,k] storage, for B about [k,n]
     d = _lib.GemmDesc(l, m, n, k, tA, tB, lda, ldb, sA, sB)
     return A2, B2, d

@@ -138,3 +138,26 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libcmk.so"))
     with pytest.raises(ImportError):
         BMMCUDA()
+
+
+def test_unaligned_operands_are_copied_to_padded_rows_when_it_pays():
+    """A large operand whose leading dimension is not a multiple of four would rule
+    out 16-byte loads in the kernels: make_desc hands over a padded copy (same
+    values, aligned pitch); small or already aligned operands are passed as they are."""
+    g = torch.Generator().manual_seed(0)
+    A = torch.randn(2, 300, 129, generator=g)            # k = 129: rows of 129 floats
+    B = torch.randn(2, 129, 301, generator=g)            # n = 301
+    A2, B2, d = _common.make_desc(A, B)
+    assert (d.lda, d.ldb, d.transA, d.transB) == (132, 304, 0, 0)
+    assert d.strideA == 300 * 132 and d.strideB == 129 * 304
+    assert torch.equal(A2, A) and torch.equal(B2, B) and A2.data_ptr() % 16 == 0
+    assert A2.stride() == (300 * 132, 132, 1)
+    # the "t" layouts keep their orientation
+    At = A.transpose(1, 2).contiguous().transpose(1, 2)  # m contiguous, m = 300 is a multiple of 4
+    Bt = B.transpose(1, 2).contiguous().transpose(1, 2)  # k contiguous, k = 129 is not
+    A3, B3, d = _common.make_desc(At, Bt)
+    assert (d.transA, d.transB, d.lda, d.ldb) == (1, 1, 300, 132)
+    assert A3.data_ptr() == At.data_ptr() and torch.equal(B3, B) and B3.stride()[1] == 1
+    # small operands are left alone
+    _, _, d = _common.make_desc(torch.zeros(1, 5, 7), torch.zeros(1, 7, 9))
+    assert (d.lda, d.ldb) == (7, 9)
