@@ -91,16 +91,15 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
     // per compare, no index registers); indices ascend with the code, so a strict
     // '<' keeps the first occurrence.  The code becomes an index once per tile.
     const int xb = xt * C::TX + wx * 64;
-    float tbest[2];
-    int tcode[2];
+    // (every search starts from +inf, not from the first product: a NaN there
+    // would lose every later comparison and hide the rest of the tile)
+    float tbest[2] = {INFINITY, INFINITY};
+    int tcode[2] = {0, 0};
     if (xb + 64 <= X.rows) {
-#pragma unroll
-      for (int by = 0; by < 2; ++by) { tbest[by] = acc[0][by][0]; tcode[by] = 0; }
 #pragma unroll
       for (int bx = 0; bx < 2; ++bx)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          if (bx == 0 && r == 0) continue;
 #pragma unroll
           for (int by = 0; by < 2; ++by) {
             const float v = acc[bx][by][r];
@@ -108,8 +107,6 @@ __global__ __launch_bounds__(kThreads, 2) void min_kernel(MinArgs a) {
           }
         }
     } else {
-#pragma unroll
-      for (int by = 0; by < 2; ++by) { tbest[by] = INFINITY; tcode[by] = 0; }
 #pragma unroll
       for (int bx = 0; bx < 2; ++bx)
 #pragma unroll

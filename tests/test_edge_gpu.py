@@ -142,6 +142,32 @@ def test_non_finite_products_min(device):
         assert (i[neg] == 333).all()
 
 
+def test_nan_products_do_not_hide_their_neighbours_in_min(device):
+    """A NaN product at any position of a tile - the first one included - loses
+    every comparison and nothing else: the minimum over the other products is
+    still found.  NaNs are planted in whole columns of B (every row of the
+    product has them) at positions that are first, last and in between for the
+    lanes of the kernel's tiles."""
+    A, B = seeded(1, 260, 1000, 16, seed=44)
+    cols = [0, 4, 31, 32, 64, 127, 128, 132, 255, 256, 511, 512, 640, 999]
+    B[0, :, cols] = float("nan")
+    C = torch.bmm(A, B)[0]
+    want_v, want_i = torch.nan_to_num(C, nan=float("inf")).min(1)
+    for mode in MODES:
+        Ad, Bd = place(A, B, mode, device)
+        v, i = MinBMMCUDA()(Ad, Bd, dim=2)
+        O.check_values(v.cpu()[0], want_v, 16, "minimum over the products that are not NaN")
+        assert torch.equal(i.cpu()[0], want_i)
+    # the same along dim=1 (NaN rows of A)
+    A2, B2 = seeded(1, 1000, 260, 16, seed=45)
+    A2[0, cols, :] = float("nan")
+    C2 = torch.bmm(A2, B2)[0]
+    want_v, want_i = torch.nan_to_num(C2, nan=float("inf")).min(0)
+    v, i = MinBMMCUDA()(A2.to(device), B2.to(device), dim=1)
+    O.check_values(v.cpu()[0], want_v, 16, "minimum over the products that are not NaN, dim=1")
+    assert torch.equal(i.cpu()[0], want_i)
+
+
 def test_non_finite_products_topk(device):
     """top-k orders by the fp32 bit pattern: +inf above every finite value, -inf
     below, NaN with a clear sign bit above +inf (torch.topk also ranks NaN
