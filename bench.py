@@ -536,6 +536,30 @@ def main():
             del cpu_args, dev_args
             torch.cuda.empty_cache()
         out["other_workloads"] = others
+    # The full record goes to stderr (and to gpurun_out/ when that exists); the one
+    # line on stdout keeps the headline in full and, per other workload, the
+    # figures only, so that it stays a few kilobytes.
+    full = json.dumps(out)
+    print(full, file=sys.stderr)
+    if os.path.isdir(os.path.join(ROOT, "gpurun_out")):
+        with open(os.path.join(ROOT, "gpurun_out", "bench_details.json"), "w") as f:
+            f.write(full + "\n")
+    if "other_workloads" in out:
+        keep = ("config", "kernel_ms", "kernel_ms_median", "frac_fp32_mfma_peak", "frac_hbm_peak",
+                "frac_valu_issue_peak")
+        brief = {}
+        for name, rec in out["other_workloads"].items():
+            b = {k: rec[k] for k in keep if k in rec}
+            if rec.get("parity") is not None:
+                b["parity_ok"] = rec["parity"]["ok"]
+            if rec.get("cpu_baseline"):
+                b["cpu_GFLOP/s"] = rec["cpu_baseline"]["value"]
+                b["cpu_cores"] = rec["cpu_baseline"]["cores"]
+            brief[name] = b
+        out["other_workloads"] = brief
+        out["other_workloads_note"] = ("shapes, step counts, parity details and CPU samples of these workloads: "
+                                       "the same record in full on stderr; kernel_ms = events around the timed "
+                                       "region / steps, after 0.3 s of warm-up")
     print(json.dumps(out))
 
 
