@@ -52,7 +52,8 @@ MEASURED_TRAFFIC = {
     "topk_bmm": ((2 * 882178 + 1.71004e6) * 1024, "profiles/topk_kernel_topk_bmm.txt"),
     "topk_bmm_k64": ((2 * 191286 + 1.70621e6) * 1024, "profiles/topk_kernel_topk_bmm_k64.txt"),
     "topk_bmm_nt": ((2 * 232602 + 499713) * 1024, "profiles/topk_kernel_topk_bmm_nt.txt"),
-    "topk_bmm_multi": ((2 * 402063 + 378880) * 1024, "profiles/topk_kernel_topk_bmm_multi.txt"),
+    "topk_bmm_multi": ((2 * 402599 + 436704) * 1024, "profiles/topk_kernel_topk_bmm_multi.txt"),
+    "topk_bmm_long_axis": ((2 * 6.02055e6 + 6.34998e6) * 1024, "profiles/topk_kernel_topk_bmm_long_axis.txt"),
     "topk_bmm_l2": ((2 * 13468.7 + 108959) * 1024, "profiles/topk_kernel_topk_bmm_l2.txt"),
     "ref_topk_bmm_32768_dim1": ((2 * 56118.1 + 77626) * 1024, "profiles/topk_kernel_ref_topk_bmm_32768_dim1.txt"),
     "derive_masks_4GiB": ((2 * 2.09725e6 + 66564) * 1024, "profiles/derive_masks_kernel_4GiB.txt"),
@@ -298,6 +299,9 @@ def make_workloads(torch, cmk, O, dev):
     # other code paths of the top-k kernel: B stored [n,k], a reduced axis of several chunks, a vector-unit distance
     topk_wl("topk_bmm_nt", 1, 262144, 1024, 256, b_transposed=True)
     topk_wl("topk_bmm_multi", 1, 16384, 16384, 256)
+    # nearest-neighbour search geometry: few kept rows, a reduced axis of hundreds of chunks
+    topk_wl("topk_bmm_long_axis", 1, 4096, 1048576, 256)
+    topk_wl("topk_bmm_long_axis_k64", 1, 16384, 131072, 64)
     topk_wl("topk_bmm_l2", 1, 65536, 1024, 64, distance="l2")
     return W
 

@@ -15,6 +15,8 @@
 //      written to the output list as (key, ~index) entries.
 // The output list is unordered; bitonic128_desc() orders it once, at the very
 // end, so that values descend and equal values come out by ascending index.
+// insert128() is the short route for a later chunk of a long axis, when the
+// list is full and few candidates beat its smallest entry.
 //
 // Replaces the reference's per-tile sort / lock / merge against a global
 // running list (kernels/topkbmm.cu:13-47, 98-183; network also in
@@ -258,6 +260,114 @@ __device__ __forceinline__ void select128(const uint32_t (&raw)[NR], IdxOf&& idx
     }
   }
   seed = lo;
+}
+
+// Folds the candidates raw[0..16) of all lanes into a FULL running list of 128
+// entries whose smallest key is `thr` (> 0), by a shorter route than
+// select128<18>: only candidates with a key above thr can enter (an equal key
+// loses the tie to the list, whose indices are lower), late chunks of a long
+// axis bring few of those, and the new threshold lies just above the old one.
+// The newcomers are compacted into `cand` (at most one per lane), the threshold
+// is searched upwards from thr over three entries per lane, and the list is
+// rewritten as its survivors followed by the surviving newcomers, both in their
+// old order, which keeps equal keys in ascending index order.  Returns false,
+// having changed nothing, when more than 64 candidates beat thr.
+template <class IdxOf>
+__device__ __forceinline__ bool insert128(const uint32_t (&raw)[16], IdxOf&& idx_of, uint32_t& thr,
+                                          entry_t* cand, entry_t* list) {
+  const int lane = threadIdx.x & 63;
+  thr = __builtin_amdgcn_readfirstlane(thr);
+  if (thr == 0xFFFFFFFFu) return true;  // nothing ranks above the list's smallest entry
+  unsigned long long m[16];
+  const int c = masks_ge(raw, thr + 1u, m);
+  if (c == 0) return true;
+  if (c > 64) return false;
+  int base = 0;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    if (m[j]) {
+      const int pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(m[j] >> 32),
+                                                __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(m[j]), base));
+      if (__builtin_amdgcn_inverse_ballot_w64(m[j])) cand[pos] = pack_entry(raw[j], idx_of(j));
+      base += __popcll(m[j]);
+    }
+  }
+  entry_t e[3];
+  uint32_t k[3];
+  e[0] = list[lane];
+  e[1] = list[lane + 64];
+  k[0] = entry_key(e[0]);
+  k[1] = entry_key(e[1]);
+  {
+    const entry_t r = cand[lane];
+    k[2] = lane < c ? raw2key(entry_key(r)) : 0u;
+    e[2] = k[2] ? (static_cast<entry_t>(k[2]) << 32) | static_cast<uint32_t>(r) : 0ull;
+  }
+  auto count3 = [&](uint32_t t) {
+    int n = 0;
+#pragma unroll
+    for (int q = 0; q < 3; ++q) n += __popcll(__ballot(k[q] >= t));
+    return n;
+  };
+  // bracket [lo, hi): count(>= lo) >= 128 > count(>= hi); hi == 0 stands for 2^32
+  uint32_t lo = thr, hi = 0;
+  int n_lo = kTop + c;
+  {
+    uint32_t t = lo, step = 1u << 13;
+    while (t < 0xFFFFFFFFu - step) {
+      t += step;
+      const int n = count3(t);
+      if (n < kTop) { hi = t; break; }
+      lo = t;
+      n_lo = n;
+      if (n == kTop) break;
+      if (step < (1u << 29)) step <<= 2;
+    }
+  }
+  while (n_lo != kTop && hi - lo != 1u) {
+    const uint32_t w = hi - lo;  // 2^32 - lo when hi == 0
+    uint32_t q = w >> 2;
+    if (q == 0) q = 1;
+    uint32_t t1 = lo + q, t2 = t1 + q, t3 = t2 + q;
+    if (t2 < t1) t2 = 0xFFFFFFFFu;
+    if (t3 < t2) t3 = 0xFFFFFFFFu;
+    int c1 = 0, c2 = 0, c3 = 0;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      c1 += __popcll(__ballot(k[r] >= t1));
+      c2 += __popcll(__ballot(k[r] >= t2));
+      c3 += __popcll(__ballot(k[r] >= t3));
+    }
+    if (c3 >= kTop) { lo = t3; n_lo = c3; }
+    else if (c2 >= kTop) { lo = t2; n_lo = c2; hi = t3; }
+    else if (c1 >= kTop) { lo = t1; n_lo = c1; hi = t2; }
+    else { hi = t1; }
+  }
+  // survivors: every entry >= lo if those are exactly 128, otherwise those above
+  // lo and then the first ones equal to lo.  Every lane holds its entries in
+  // registers by now (the ballots above needed them), so the list can be
+  // rewritten in place.
+  const bool exact = n_lo == kTop;
+  int pos = 0;
+#pragma unroll
+  for (int q = 0; q < 3; ++q) {
+    const bool g = exact ? k[q] >= lo : k[q] > lo;
+    const unsigned long long mq = __ballot(g);
+    if (g) list[pos + prefix_in(mq)] = e[q];
+    pos += __popcll(mq);
+  }
+  if (!exact) {
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+      const bool tie = k[q] == lo;
+      const unsigned long long mq = __ballot(tie);
+      const int p = pos + prefix_in(mq);
+      if (tie && p < kTop) list[p] = e[q];
+      pos += __popcll(mq);
+    }
+  }
+  thr = lo;
+  return true;
 }
 
 // Value of `v` in lane (lane ^ STRIDE).

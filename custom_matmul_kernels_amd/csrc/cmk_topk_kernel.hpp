@@ -55,11 +55,15 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
   constexpr int stageFloats = kPassRows * kStagePitch;
   constexpr int listFloats = kStripRows * kTop * 2;
   constexpr int listAt = MULTI ? (C::ldsFloats > stageFloats ? C::ldsFloats : stageFloats) : stageFloats;
-  constexpr int selFloats = listAt + listFloats > C::ldsFloats ? listAt + listFloats : C::ldsFloats;
+  // MULTI: behind the lists, the smallest key of every row's list once it is full
+  constexpr int thrAt = listAt + listFloats;
+  constexpr int endFloats = thrAt + (MULTI ? kStripRows : 0);
+  constexpr int selFloats = endFloats > C::ldsFloats ? endFloats : C::ldsFloats;
   static_assert(selFloats * 4 <= 160 * 1024, "LDS capacity");
   __shared__ __attribute__((aligned(16))) float lds[selFloats];
   // running top-128 of every row of the strip
   entry_t(*list)[kTop] = reinterpret_cast<entry_t(*)[kTop]>(lds + listAt);
+  uint32_t* const row_thr = reinterpret_cast<uint32_t*>(lds + thrAt);
 
 
   // the previous row's threshold seeds the next search; it carries over from
@@ -172,28 +176,36 @@ __global__ __launch_bounds__(kTopkThreads, 1) void topk_kernel(TopkArgs a) {
         if (y0 + r >= Yext) continue;
         const float* src = lds + pr * kStagePitch;
         const int xl = xc0 + lane;
-        uint32_t key[18];  // fp32 bit patterns
+        uint32_t k16[16];  // fp32 bit patterns
         if (xc0 + 1024 <= x_limit) {
 #pragma unroll
-          for (int j = 0; j < 16; ++j) key[j] = __float_as_uint(src[lane + 64 * j]);
+          for (int j = 0; j < 16; ++j) k16[j] = __float_as_uint(src[lane + 64 * j]);
         } else {
 #pragma unroll
           for (int j = 0; j < 16; ++j)
-            key[j] = xl + 64 * j < x_limit ? __float_as_uint(src[lane + 64 * j]) : kNoCandidate;
+            k16[j] = xl + 64 * j < x_limit ? __float_as_uint(src[lane + 64 * j]) : kNoCandidate;
         }
         if (!MULTI || xt0 == xt_begin) {
           // first chunk: the running list is empty
-          uint32_t k16[16];
-#pragma unroll
-          for (int j = 0; j < 16; ++j) k16[j] = key[j];
           select128<16>(k16, [&](int j) { return xl + 64 * j; }, seed, cand, list[r]);
+          if constexpr (MULTI) row_thr[r] = seed;
         } else {
-          const entry_t e0 = list[r][lane], e1 = list[r][lane + 64];
-          key[16] = key2raw(entry_key(e0));
-          key[17] = key2raw(entry_key(e1));
-          const int ri0 = entry_idx(e0), ri1 = entry_idx(e1);
-          select128<18>(key, [&](int j) { return j < 16 ? xl + 64 * j : (j == 16 ? ri0 : ri1); },
-                        seed, cand, list[r]);
+          // a full list takes the few candidates that beat its smallest entry by
+          // the short route; otherwise list and chunk are selected from together
+          uint32_t thr = row_thr[r];
+          if (thr == 0u || !insert128(k16, [&](int j) { return xl + 64 * j; }, thr, cand, list[r])) {
+            uint32_t key[18];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) key[j] = k16[j];
+            const entry_t e0 = list[r][lane], e1 = list[r][lane + 64];
+            key[16] = key2raw(entry_key(e0));
+            key[17] = key2raw(entry_key(e1));
+            const int ri0 = entry_idx(e0), ri1 = entry_idx(e1);
+            select128<18>(key, [&](int j) { return j < 16 ? xl + 64 * j : (j == 16 ? ri0 : ri1); },
+                          seed, cand, list[r]);
+            thr = seed;
+          }
+          row_thr[r] = thr;
         }
       }
     }

@@ -85,6 +85,39 @@ def test_ties_at_the_threshold_keep_the_lowest_indices_across_chunks(device):
     assert torch.equal(i.cpu(), torch.cat([hot3.sort().values, torch.from_numpy(rest)]))
 
 
+def test_long_reduced_axis_with_exact_products_matches_a_stable_sort(device):
+    """Forty chunks of candidates per row, products that are small integers
+    (exact in fp32, full of ties): the result must be the first 128 of a stable
+    descending sort, i.e. equal values by ascending index.  The patterns make
+    late chunks bring no newcomer (descending ramp), only newcomers (ascending
+    ramp), a few (random digits) and ties with the list's smallest entry."""
+    N = 40000
+    gen = torch.Generator().manual_seed(23)
+    ramps = {
+        "digits": torch.randint(0, 10, (N,), generator=gen).float(),
+        "ascending": torch.arange(N).float(),
+        "descending": torch.arange(N, 0, -1).float(),
+        "steps": (torch.arange(N) // 300).float(),
+        "sawtooth": (torch.arange(N) % 1500).float(),
+        "rare": (torch.rand(N, generator=gen) < 0.002).float() * torch.randint(1, 4, (N,), generator=gen).float(),
+    }
+    scale = torch.tensor([1.0, -1.0, 2.0, -3.0, 0.0]).repeat(14)[:68]      # 68 rows: two strips, the second ragged
+    for name, b in ramps.items():
+        say("long axis", name)
+        A = scale.view(1, -1, 1).clone()
+        B = b.view(1, 1, N).clone()
+        C = torch.bmm(A, B)
+        want = C.sort(dim=2, descending=True, stable=True)
+        v, i = TopkBMMCUDA()(A.to(device), B.to(device), k=128, dim=2)
+        assert torch.equal(v.cpu(), want.values[..., :128]), name
+        assert torch.equal(i.cpu(), want.indices[..., :128]), name
+        # the same products with the long axis first (dim=1), cut into splits and merged
+        v, i = TopkBMMCUDA()(B.transpose(1, 2).contiguous().to(device), A.transpose(1, 2).contiguous().to(device),
+                             k=128, dim=1)
+        assert torch.equal(v.cpu(), want.values[..., :128]), name + " dim=1"
+        assert torch.equal(i.cpu(), want.indices[..., :128]), name + " dim=1"
+
+
 # ------------------------------------------------ empty / short axes --------
 def test_topk_over_an_empty_or_short_reduced_axis(device):
     op = TopkBMMCUDA()
@@ -273,7 +306,7 @@ def test_mbmm_layouts_match_oracle(device, shape, mode, share):
 def _dims(rng):
     L = rng.choice([1, 1, 2, 3, 40])
     M = rng.choice([1, 7, 64, 100, 128, 129, 255, 256, 300, 513, 640, 1500])
-    N = rng.choice([1, 5, 64, 96, 128, 130, 256, 384, 500, 1024, 1100, 2500])
+    N = rng.choice([1, 5, 64, 96, 128, 130, 256, 384, 500, 1024, 1100, 2500, 9000])
     K = rng.choice([1, 3, 8, 31, 32, 33, 36, 64, 65, 96, 100, 128, 160, 200, 257])
     if L == 40 and M * N * K > 3e7:
         L = 4
