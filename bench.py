@@ -285,6 +285,7 @@ def make_workloads(torch, cmk, O, dev):
     # the shapes the reference publishes numbers for (its notebooks' printed results and plots, Tesla T4)
     bmm_wl("ref_bmm_8192x512", 1, 8192, 8192, 512)             # colab/test_bmm.ipynb:2163-2164
     bmm_wl("ref_bmm_8192_cube", 1, 8192, 8192, 8192)           # imgs/bmm_A[1,N,N] B[1,N,N].png
+    bmm_wl("bmm_long_k", 1, 512, 512, 4096)                    # few tiles, long contraction: k cut into ranges
     min_wl("ref_min_bmm_1024x131072_k64", 1, 1024, 131072, 64)  # colab/test_minbmm.ipynb:2192-2193
     min_wl("ref_min_bmm_16384_k64", 1, 16384, 16384, 64)       # imgs/min_bmm_A[1,N,64] B[1,64,N].png
     min_wl("ref_min_bmm_16384_k256", 1, 16384, 16384, 256)     # imgs/min_bmm_A[1,N,256] B[1,256,N].png

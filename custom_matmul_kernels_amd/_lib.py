@@ -23,6 +23,7 @@ ERR_INVALID_ARG, ERR_UNSUPPORTED, ERR_WORKSPACE = -1, -2, -3
 # every symbol include/cmk.h declares
 EXPORTS = (
     "cmk_bmm_f32",
+    "cmk_bmm_ws_f32",
     "cmk_mbmm_f32",
     "cmk_derive_masks_u8",
     "cmk_min_bmm_f32",
@@ -91,13 +92,14 @@ def load():
     p, i, sz, ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_longlong
     dp = ctypes.POINTER(GemmDesc)
     lib.cmk_bmm_f32.argtypes = [p, p, p, dp, p]
+    lib.cmk_bmm_ws_f32.argtypes = [p, p, p, dp, p, sz, p]
     lib.cmk_mbmm_f32.argtypes = [p, p, p, p, p, p, i, dp, p]
     lib.cmk_derive_masks_u8.argtypes = [p, p, p, i, i, i, p]
     lib.cmk_min_bmm_f32.argtypes = [p, p, p, p, dp, i, i, p, sz, p]
     lib.cmk_min_bmm_f32_static.argtypes = [p, p, p, p, dp, i, i, p]
     lib.cmk_topk_bmm_f32.argtypes = [p, p, p, p, dp, i, i, i, p, sz, p]
     lib.cmk_topk_1d_f32.argtypes = [p, ll, p, p, i, p, sz, p]
-    for name in ("cmk_bmm_f32", "cmk_mbmm_f32", "cmk_derive_masks_u8", "cmk_min_bmm_f32", "cmk_min_bmm_f32_static",
+    for name in ("cmk_bmm_f32", "cmk_bmm_ws_f32", "cmk_mbmm_f32", "cmk_derive_masks_u8", "cmk_min_bmm_f32", "cmk_min_bmm_f32_static",
                  "cmk_topk_bmm_f32", "cmk_topk_1d_f32"):
         getattr(lib, name).restype = i
     lib.cmk_workspace_bytes.argtypes = [i, i, i, i, i, i]

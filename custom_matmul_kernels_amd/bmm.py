@@ -39,9 +39,13 @@ class BMMCUDA:
         C = torch.empty([l, m, n], device=A.device, dtype=A.dtype)
         if C.numel():
             A2, B2, desc = _common.make_desc(A, B)
+            # few tiles and a long contraction: the library cuts k into ranges
+            # and asks for room for their partial products
+            ws, ws_bytes = _common.workspace(_lib.OP_BMM, l, m, n, k, 0, A.device)
             with torch.cuda.device(A.device):
-                _lib.check(self._lib.cmk_bmm_f32(
+                _lib.check(self._lib.cmk_bmm_ws_f32(
                     A2.data_ptr(), B2.data_ptr(), C.data_ptr(), desc,
+                    ws.data_ptr() if ws is not None else None, ws_bytes,
                     _common.stream_ptr(A.device)))
         if two_dimensional:
             C = C[0]

@@ -60,6 +60,7 @@ int compute_units() {
   return cached_cus;
 }
 
+size_t bmm_workspace_bytes(int L, int M, int N, int K);
 size_t min_workspace_bytes(int L, int Xext, int Yext, int K);
 size_t topk_workspace_bytes(int L, int Xext, int Yext, int K);
 size_t topk1d_workspace_bytes(long long n);
@@ -69,6 +70,8 @@ size_t topk1d_workspace_bytes(long long n);
 extern "C" size_t cmk_workspace_bytes(int op, int L, int M, int N, int K, int dim) {
   if (L < 0 || M < 0 || N < 0) return 0;
   switch (op) {
+    case CMK_OP_BMM:
+      return cmk::bmm_workspace_bytes(L, M, N, K);
     case CMK_OP_MIN_BMM:
       if (dim != 1 && dim != 2) return 0;
       return cmk::min_workspace_bytes(L, dim == 2 ? N : M, dim == 2 ? M : N, K);

@@ -22,6 +22,10 @@ struct BmmArgs {
   int run;           // consecutive tiles along m per work-group
   int mask_batched;  // 1: masks have a leading batch axis, 0: shared by all batches
   int vecA, vecB;
+  // contraction cut into `ksplits` ranges of `klen` (a multiple of the slab depth):
+  // the launch then has L * ksplits "batches", batch b * ksplits + j holds the
+  // partial product of range j of batch b, and C is the workspace of partials
+  int ksplits, klen;
 };
 
 constexpr int kMaskRows = 128;    // element-mask tile staged in LDS: rows ...
@@ -87,9 +91,19 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
 
   Operand X{uniform_ptr(a.A + (long long)b * a.strideA), a.lda, a.M, a.vecA};
   Operand Y{uniform_ptr(a.B + (long long)b * a.strideB), a.ldb, a.N, a.vecB};
+  int K = a.K;
+  if constexpr (!MASKED) {
+    if (a.ksplits > 1) {
+      const int bb = b / a.ksplits;
+      const int k0 = (b - bb * a.ksplits) * a.klen;
+      K = min(a.klen, a.K - k0);
+      X.p = uniform_ptr(a.A + (long long)bb * a.strideA + (XK == KC ? (long long)k0 : (long long)k0 * a.lda));
+      Y.p = uniform_ptr(a.B + (long long)bb * a.strideB + (YK == KC ? (long long)k0 : (long long)k0 * a.ldb));
+    }
+  }
 
   C core;
-  core.begin(X, Y, tile_m0 * C::TX, n0, a.K, ntiles, lds);
+  core.begin(X, Y, tile_m0 * C::TX, n0, K, ntiles, lds);
   for (int ti = 0; ti < ntiles; ++ti) {
     // the dense product starts its accumulators from a literal zero; for the
     // masked one that form measured slower (191 vs 165 us at the benchmark shape)
@@ -263,9 +277,81 @@ static BmmArgs make_args(const float* A, const float* B, float* C, const cmk_gem
   return a;
 }
 
+// Long contractions with few tiles: how many ranges the contraction is cut into
+// so that the chip has work (each range at least four slabs), and their length.
+static int plan_bmm_ksplits(int L, int M, int N, int K, int* klen) {
+  const long long tiles = (long long)L * ((M + 63) / 64) * ((N + 63) / 64);
+  const int slabs = (K + 31) / 32;
+  *klen = K;
+  if (tiles == 0 || slabs < 8) return 1;
+  // one 64x64 work-group per CU: more ranges than that measured slower (the sum
+  // reads every partial once more), fewer leave CUs idle
+  long long want = (compute_units() + tiles - 1) / tiles;
+  if (want > slabs / 4) want = slabs / 4;
+  if (want > 64) want = 64;
+  if (want < 2) return 1;
+  const int per = (slabs + (int)want - 1) / (int)want;
+  *klen = per * 32;
+  return (slabs + per - 1) / per;
+}
+
+size_t bmm_workspace_bytes(int L, int M, int N, int K) {
+  int klen;
+  const int s = plan_bmm_ksplits(L, M, N, K, &klen);
+  return s > 1 ? (size_t)s * L * M * N * sizeof(float) : 0;
+}
+
+// C[b][e] = sum over j, in ascending j, of part[b * s + j][e]; `mn` elements per
+// matrix.  V = 4 when everything can move as 16-byte vectors.
+template <int V>
+__global__ __launch_bounds__(256) void bmm_sum_kernel(const float* __restrict__ part, float* __restrict__ C,
+                                                      long long mn, long long total, int s) {
+  typedef float vec_t __attribute__((ext_vector_type(V)));
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i * V < total; i += stride) {
+    const long long o = i * V;
+    const long long b = o / mn, e = o - b * mn;
+    const float* p = part + (b * s) * mn + e;
+    vec_t acc = *reinterpret_cast<const vec_t*>(p);
+    for (int j = 1; j < s; ++j) acc += *reinterpret_cast<const vec_t*>(p + j * mn);
+    *reinterpret_cast<vec_t*>(C + o) = acc;
+  }
+}
+
 }  // namespace cmk
 
 using namespace cmk;
+
+extern "C" int cmk_bmm_ws_f32(const float* A, const float* B, float* C, const cmk_gemm_desc* d,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+  if (int e = check_desc(d)) return e;
+  if (d->L == 0 || d->M == 0 || d->N == 0) return CMK_OK;
+  int klen;
+  const int s = plan_bmm_ksplits(d->L, d->M, d->N, d->K, &klen);
+  if (s <= 1) return cmk_bmm_f32(A, B, C, d, stream);
+  if (!C || !A || !B) return fail(CMK_ERR_INVALID_ARG, "cmk_bmm_ws_f32: null pointer");
+  const size_t need = (size_t)s * d->L * d->M * d->N * sizeof(float);
+  if (!workspace || workspace_bytes < need)
+    return fail(CMK_ERR_WORKSPACE, "cmk_bmm_ws_f32: workspace of %zu bytes required, %zu given", need,
+                workspace_bytes);
+  BmmArgs a = make_args(A, B, static_cast<float*>(workspace), d, 64);
+  a.ksplits = s;
+  a.klen = klen;
+  a.L = d->L * s;
+  if (int e = check_grid((long long)a.L * a.tiles_m * a.tiles_n)) return e;
+  hipStream_t st = (hipStream_t)stream;
+  if (int e = hip_status(launch_bmm<false, 1>(a, d->transA, d->transB, st), "cmk_bmm_ws_f32 launch")) return e;
+  const long long mn = (long long)d->M * d->N, total = mn * d->L;
+  const bool vec = (mn & 3) == 0 && ((reinterpret_cast<uintptr_t>(workspace) | reinterpret_cast<uintptr_t>(C)) & 15) == 0;
+  const long long items = vec ? total / 4 : total;
+  long long blocks = (items + 255) / 256;
+  if (blocks > 8ll * compute_units()) blocks = 8ll * compute_units();
+  if (vec) hipLaunchKernelGGL(bmm_sum_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, st,
+                              static_cast<const float*>(workspace), C, mn, total, s);
+  else hipLaunchKernelGGL(bmm_sum_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, st,
+                          static_cast<const float*>(workspace), C, mn, total, s);
+  return hip_status(hipGetLastError(), "cmk_bmm_ws_f32 sum launch");
+}
 
 extern "C" int cmk_bmm_f32(const float* A, const float* B, float* C, const cmk_gemm_desc* d,
                            void* stream) {

@@ -73,6 +73,24 @@ int cmk_bmm_f32(const float* A, const float* B, float* C,
                 const cmk_gemm_desc* d, void* stream);
 
 /*
+ * The same product for callers that can lend a workspace of
+ * cmk_workspace_bytes(CMK_OP_BMM, L, M, N, K, 0) bytes.  When C has too few
+ * tiles to occupy the GPU and the contraction is long (say 512x512 with
+ * K = 4096), the contraction is cut into ranges whose partial products go to
+ * the workspace and are summed in ascending order of k by a second kernel:
+ * results are reproducible from run to run, and differ from cmk_bmm_f32's by
+ * fp32 rounding only.  With a workspace size of 0 reported, or given, for
+ * shapes that need none, this is cmk_bmm_f32.  The reference walks the whole
+ * contraction in one block per tile (kernels/bmm.cu:184-274) and has no
+ * counterpart; the Python class calls this entry point (reference
+ * bmm.py:68-129 allocates its result through PyTorch at every call, as this
+ * workspace is).
+ */
+int cmk_bmm_ws_f32(const float* A, const float* B, float* C,
+                   const cmk_gemm_desc* d,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Masked product: C = (A@B) * element_mask where the 128x128 tile's
  * block_mask and the 8x8 micro-tile's thread_mask are both non-zero, else 0.
  * Tiles whose block_mask is 0 are not computed (only zeros are written).

@@ -50,6 +50,64 @@ def test_bmm_matches_oracle(device, shape, mode):
     O.check_values(C.cpu(), torch.from_numpy(O.c_bmm(A.numpy(), B.numpy())), K, "bmm")
 
 
+# few tiles and a long contraction: k is cut into ranges whose partial products go
+# to a workspace and are summed by a second kernel
+BMM_LONG_K = [(1, 200, 136, 1000), (3, 129, 257, 517), (1, 64, 64, 4099), (2, 300, 70, 2048), (1, 1, 1, 300)]
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("shape", BMM_LONG_K)
+def test_bmm_long_contraction_few_tiles(device, shape, mode):
+    from custom_matmul_kernels_amd import _lib
+    say("bmm long k", shape, mode)
+    L, M, N, K = shape
+    lib = _lib.load()
+    assert lib.cmk_workspace_bytes(_lib.OP_BMM, L, M, N, K, 0) > 0
+    A, B = seeded(L, M, N, K, seed=2, dist="uniform")
+    Ad, Bd = place(A, B, mode, device)
+    op = BMMCUDA()
+    C = op(Ad, Bd)
+    O.check_values(C.cpu(), torch.from_numpy(O.c_bmm(A.numpy(), B.numpy())), K, "bmm long k")
+    assert torch.equal(C, op(Ad, Bd)), "two runs differ"
+    # small integers: every partial sum is exact, so the cut must not show
+    gen = torch.Generator().manual_seed(K)
+    Ai = torch.randint(-3, 4, (L, M, K), generator=gen).float()
+    Bi = torch.randint(-3, 4, (L, K, N), generator=gen).float()
+    Aid, Bid = place(Ai, Bi, mode, device)
+    assert torch.equal(op(Aid, Bid).cpu(), torch.bmm(Ai.double(), Bi.double()).float())
+
+
+def test_bmm_workspace_entry_point_through_the_abi(device):
+    """cmk_bmm_ws_f32 against cmk_bmm_f32 on the same operands: equal within fp32
+    rounding where k is cut, bit-equal where it is not; too small a workspace is
+    refused with a message and nothing is launched."""
+    from custom_matmul_kernels_amd import _lib
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(device).cuda_stream
+    for (L, M, N, K) in [(1, 256, 256, 2048), (2, 100, 90, 700), (4, 512, 512, 512)]:
+        say("bmm ws abi", (L, M, N, K))
+        A, B = seeded(L, M, N, K, seed=5, dist="uniform")
+        Ad, Bd = A.to(device), B.to(device)
+        d = _lib.GemmDesc(L, M, N, K, 0, 0, K, N, M * K, K * N)
+        plain = torch.full((L, M, N), float("nan"), device=device)
+        _lib.check(lib.cmk_bmm_f32(Ad.data_ptr(), Bd.data_ptr(), plain.data_ptr(), d, stream))
+        need = lib.cmk_workspace_bytes(_lib.OP_BMM, L, M, N, K, 0)
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=device)
+        cut = torch.full((L, M, N), float("nan"), device=device)
+        _lib.check(lib.cmk_bmm_ws_f32(Ad.data_ptr(), Bd.data_ptr(), cut.data_ptr(), d, ws.data_ptr(), need, stream))
+        torch.cuda.synchronize()
+        if need == 0:
+            assert torch.equal(cut, plain)
+        else:
+            O.check_values(cut.cpu(), plain.cpu(), K, "bmm ws against plain")
+            untouched = torch.full((L, M, N), 7.0, device=device)
+            rc = lib.cmk_bmm_ws_f32(Ad.data_ptr(), Bd.data_ptr(), untouched.data_ptr(), d, ws.data_ptr(), need - 1,
+                                    stream)
+            torch.cuda.synchronize()
+            assert rc == _lib.ERR_WORKSPACE and b"workspace" in lib.cmk_last_error()
+            assert (untouched == 7.0).all()
+
+
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("name", INT_CASES)
 def test_bmm_integer_cases_are_bit_exact(device, name, mode):
