@@ -284,9 +284,15 @@ static int plan_bmm_ksplits(int L, int M, int N, int K, int* klen) {
   const int slabs = (K + 31) / 32;
   *klen = K;
   if (tiles == 0 || slabs < 8) return 1;
-  // one 64x64 work-group per CU: more ranges than that measured slower (the sum
-  // reads every partial once more), fewer leave CUs idle
-  long long want = (compute_units() + tiles - 1) / tiles;
+  // Up to half a chip of tiles: one 64x64 work-group per CU (more ranges measured
+  // slower: the sum reads every partial once more; fewer leave CUs idle).  Up to
+  // a whole chip: four ranges, so that every SIMD has waves to switch between,
+  // once the contraction is long enough to pay for the second kernel (measured:
+  // from about 48 slabs).
+  const long long cus = compute_units();
+  long long want;
+  if (tiles * 2 > cus) want = (tiles <= cus && slabs >= 48) ? 4 : 1;
+  else want = (cus + tiles - 1) / tiles;
   if (want > slabs / 4) want = slabs / 4;
   if (want > 64) want = 64;
   if (want < 2) return 1;
