@@ -46,8 +46,8 @@ PEAK_VALU_TOPS = 39.3           # 256 CUs x 64 lanes x 2.4 GHz: one fp32 vector 
 MEASURED_TRAFFIC = {
     "min_bmm_large": ((2 * 2.12432e6 + 2048) * 1024, "profiles/min_kernel_min_bmm_large.txt"),
     "min_bmm_small": ((2 * 4711.57 + 512) * 1024, "profiles/min_kernel_min_bmm_small.txt"),
-    "bmm": ((2 * 65926.9 + 524291) * 1024, "profiles/bmm_kernel_bmm.txt"),
-    "mbmm": ((2 * 48340 + 524291) * 1024, "profiles/bmm_kernel_mbmm.txt"),
+    "bmm": ((2 * 65882.2 + 524304) * 1024, "profiles/bmm_kernel_bmm.txt"),
+    "mbmm": ((2 * 48379.7 + 524289) * 1024, "profiles/bmm_kernel_mbmm.txt"),
     "ref_mbmm_tril_1024": ((2 * 70793.2 + 524290) * 1024, "profiles/bmm_kernel_ref_mbmm_tril_1024.txt"),
     "topk_bmm": ((2 * 882178 + 1.71004e6) * 1024, "profiles/topk_kernel_topk_bmm.txt"),
     "topk_bmm_k64": ((2 * 191286 + 1.70621e6) * 1024, "profiles/topk_kernel_topk_bmm_k64.txt"),
