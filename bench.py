@@ -38,26 +38,63 @@ PEAK_HBM_GBS = 8000.0
 PEAK_VALU_TOPS = 39.3           # 256 CUs x 64 lanes x 2.4 GHz: one fp32 vector instruction per lane and cycle
                                 # (packed fp32 is switched off in this build)
 
-# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc
-# (FETCH_SIZE, WRITE_SIZE: KiB per dispatch).  On this box FETCH_SIZE reads half
-# of the true bytes of a plain 1 GiB device copy and WRITE_SIZE all of them, so
-# traffic = (2 * FETCH_SIZE + WRITE_SIZE) * 1024.  The counters cannot be read
-# from inside this process; each figure names the summary it was taken from.
-MEASURED_TRAFFIC = {
-    "min_bmm_large": ((2 * 2.12432e6 + 2048) * 1024, "profiles/min_kernel_min_bmm_large.txt"),
-    "min_bmm_small": ((2 * 4711.57 + 512) * 1024, "profiles/min_kernel_min_bmm_small.txt"),
-    "bmm": ((2 * 65882.2 + 524304) * 1024, "profiles/bmm_kernel_bmm.txt"),
-    "mbmm": ((2 * 48379.7 + 524289) * 1024, "profiles/bmm_kernel_mbmm.txt"),
-    "ref_mbmm_tril_1024": ((2 * 70793.2 + 524290) * 1024, "profiles/bmm_kernel_ref_mbmm_tril_1024.txt"),
-    "topk_bmm": ((2 * 882178 + 1.71004e6) * 1024, "profiles/topk_kernel_topk_bmm.txt"),
-    "topk_bmm_k64": ((2 * 191286 + 1.70621e6) * 1024, "profiles/topk_kernel_topk_bmm_k64.txt"),
-    "topk_bmm_nt": ((2 * 232602 + 499713) * 1024, "profiles/topk_kernel_topk_bmm_nt.txt"),
-    "topk_bmm_multi": ((2 * 402599 + 436704) * 1024, "profiles/topk_kernel_topk_bmm_multi.txt"),
-    "topk_bmm_long_axis": ((2 * 6.02055e6 + 6.34998e6) * 1024, "profiles/topk_kernel_topk_bmm_long_axis.txt"),
-    "topk_bmm_l2": ((2 * 13468.7 + 108959) * 1024, "profiles/topk_kernel_topk_bmm_l2.txt"),
-    "ref_topk_bmm_32768_dim1": ((2 * 56118.1 + 77626) * 1024, "profiles/topk_kernel_ref_topk_bmm_32768_dim1.txt"),
-    "derive_masks_4GiB": ((2 * 2.09725e6 + 66564) * 1024, "profiles/derive_masks_kernel_4GiB.txt"),
-}
+# HBM-side bytes per launch of the dominant kernel come from the tracked
+# rocprofv3 summaries under profiles/ (FETCH_SIZE, WRITE_SIZE: KiB per dispatch):
+# the counters cannot be read from inside this process, so the file of a workload
+# (profiles/<kernel>_<workload>.txt) is parsed at start-up and every figure names
+# the file it was read from.  On this box FETCH_SIZE reads half of the true bytes
+# of a plain 1 GiB device copy and WRITE_SIZE all of them
+# (profiles/copy_probe_1GiB.txt), so traffic = (2 * FETCH_SIZE + WRITE_SIZE) * 1024.
+PROFILES_DIR = os.path.join(ROOT, "profiles")
+
+
+def profile_of(name):
+    """(path relative to the repository, kernel tag) of the summary of workload `name`, or None."""
+    try:
+        files = sorted(os.listdir(PROFILES_DIR))
+    except OSError:
+        return None
+    tail = "_" + name + ".txt"
+    for f in files:
+        if f.endswith(tail) and f[:len(f) - len(tail)].endswith("_kernel"):
+            return os.path.join("profiles", f), f[:len(f) - len(tail)]
+    return None
+
+
+def measured_traffic(name):
+    """(bytes per launch of the dominant kernel, file, {kernel: avg microseconds per launch}) from the
+    tracked summary of workload `name`; (None, None, {}) when there is none."""
+    found = profile_of(name)
+    if not found:
+        return None, None, {}
+    path, tag = found
+    fetch = write = None
+    trace = {}
+    in_trace = False
+    with open(os.path.join(ROOT, path)) as f:
+        for line in f:
+            t = line.split()
+            if line.startswith("Kernel trace"):
+                in_trace = True
+                continue
+            if line.startswith("Counters"):
+                in_trace = False
+            if in_trace and len(t) >= 6 and "cmk::" in line and t[-1].endswith("%"):
+                kernel = line[:line.rindex(t[-5])].strip()     # calls avg min max time%
+                trace[kernel] = float(t[-4])
+            if "cmk::" + tag not in line:
+                continue
+            for key in ("FETCH_SIZE", "WRITE_SIZE"):
+                if key in t and t[-1].startswith("avg="):
+                    v = float(t[-1][4:])
+                    if key == "FETCH_SIZE":
+                        fetch = v
+                    else:
+                        write = v
+    if fetch is None or write is None:
+        return None, path, trace
+    return (2 * fetch + write) * 1024, path, trace
+
 
 SEED = 0
 WARM_SECONDS = 0.3              # warm-up of the short workloads
@@ -406,7 +443,7 @@ def parity_of(torch, wl, cpu_args, dev_args):
 
 
 def roofline_of(name, wl, kern_ms):
-    traffic, source = MEASURED_TRAFFIC.get(name, (None, None))
+    traffic, source, _ = measured_traffic(name)
     if wl["flop"] == 0:
         ach = wl["bytes"] / (kern_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -426,6 +463,8 @@ def roofline_of(name, wl, kern_ms):
     roof["traffic"] = traffic
     if source:
         roof["traffic_source"] = source
+    if traffic and wl.get("bytes"):
+        roof["traffic_over_algorithmic_bytes"] = round(traffic / wl["bytes"], 2)
     roof["kernel_ms"] = round(kern_ms, 5)
     return roof
 
@@ -518,21 +557,36 @@ def main():
                    "kernel_ms": round(kern_o, 5), "kernel_ms_median": round(med_o, 5)}
             if "config" in w:
                 rec["config"] = w["config"]
-            if w["flop"] > 0:
+            traffic, source, trace = measured_traffic(name)
+            strict_ms = max(kern_o, med_o)       # the less favourable of the two live clocks
+            if w.get("mbmm"):
+                # skipped tiles do no arithmetic: only the executed work is priced against the matrix peak
+                kept = int(dev_args[2].sum())
+                rec["kept_tiles"] = kept
+                executed = 2.0 * 128 * 128 * cpu_args[0].shape[2] * kept
+                rec["dense_equivalent_GFLOP/s"] = round(w["flop"] / (kern_o * 1e-3) / 1e9, 1)
+                rec["executed_GFLOP/s"] = round(executed / (kern_o * 1e-3) / 1e9, 1)
+                rec["executed_frac_fp32_mfma_peak"] = round(executed / (kern_o * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)
+            elif w["flop"] > 0:
                 rec["GFLOP/s"] = round(w["flop"] / (kern_o * 1e-3) / 1e9, 1)
-                if "valu_ops" in w:
-                    rec["frac_valu_issue_peak"] = round(w["valu_ops"] / (kern_o * 1e-3) / 1e12 / PEAK_VALU_TOPS, 4)
-                else:
-                    rec["frac_fp32_mfma_peak"] = round(w["flop"] / (kern_o * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)
+                key = "frac_valu_issue_peak" if "valu_ops" in w else "frac_fp32_mfma_peak"
+                work = w["valu_ops"] / PEAK_VALU_TOPS if "valu_ops" in w else w["flop"] / PEAK_FP32_MFMA_TFLOPS
+                # priced by the stricter clock; the region average is carried beside it
+                rec[key] = round(work / (strict_ms * 1e-3) / 1e12, 4)
+                rec[key + "_region_average"] = round(work / (kern_o * 1e-3) / 1e12, 4)
+                if len(trace) > 1:
+                    # an operation of several launches: the kernels' own durations from the tracked trace
+                    rec["trace_us"] = {k: v for k, v in trace.items()}
+                    rec[key + "_by_trace"] = round(work / (sum(trace.values()) * 1e-6) / 1e12, 4)
             if "bytes" in w:
                 rec["GB/s"] = round(w["bytes"] / (kern_o * 1e-3) / 1e9, 1)
                 rec["frac_hbm_peak"] = round(rec["GB/s"] / PEAK_HBM_GBS, 4)
-            if name in MEASURED_TRAFFIC:
-                rec["traffic"], rec["traffic_source"] = MEASURED_TRAFFIC[name]
-            if w.get("mbmm"):
-                kept = int(dev_args[2].sum())
-                rec["kept_tiles"] = kept
-                rec["executed_GFLOP/s"] = round(2.0 * 128 * 128 * cpu_args[0].shape[2] * kept / (kern_o * 1e-3) / 1e9, 1)
+            if traffic:
+                rec["traffic"], rec["traffic_source"] = traffic, source
+                if w.get("bytes"):
+                    rec["traffic_over_algorithmic_bytes"] = round(traffic / w["bytes"], 2)
+                    # what actually moved, by the counters, over the live time
+                    rec["frac_hbm_peak_by_counter_bytes"] = round(traffic / (kern_o * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
             if not a.no_parity:
                 rec["parity"] = parity_of(torch, w, cpu_args, dev_args)
             if not a.no_cpu and "cpu" in w:
@@ -550,8 +604,9 @@ def main():
         with open(os.path.join(ROOT, "gpurun_out", "bench_details.json"), "w") as f:
             f.write(full + "\n")
     if "other_workloads" in out:
-        keep = ("config", "kernel_ms", "kernel_ms_median", "frac_fp32_mfma_peak", "frac_hbm_peak",
-                "frac_valu_issue_peak")
+        keep = ("config", "kernel_ms", "kernel_ms_median", "frac_fp32_mfma_peak", "frac_fp32_mfma_peak_region_average",
+                "frac_fp32_mfma_peak_by_trace", "executed_frac_fp32_mfma_peak", "frac_hbm_peak",
+                "frac_hbm_peak_by_counter_bytes", "frac_valu_issue_peak", "traffic_over_algorithmic_bytes")
         brief = {}
         for name, rec in out["other_workloads"].items():
             b = {k: rec[k] for k in keep if k in rec}
@@ -564,7 +619,9 @@ def main():
         out["other_workloads"] = brief
         out["other_workloads_note"] = ("shapes, step counts, parity details and CPU samples of these workloads: "
                                        "the same record in full on stderr; kernel_ms = events around the timed "
-                                       "region / steps, after 0.3 s of warm-up")
+                                       "region / steps, after 0.3 s of warm-up; fractions are priced by the larger of "
+                                       "kernel_ms and kernel_ms_median (the region average is carried beside them); "
+                                       "mbmm: only the kept tiles' arithmetic counts")
     print(json.dumps(out))
 
 

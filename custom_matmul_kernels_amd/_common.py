@@ -70,20 +70,27 @@ ALIGN_COPY_MAX = 1 << 28
 def _aligned(T, trans, ld, stride):
     """The operand itself when the kernels can fetch it with 16-byte loads (or
     when a copy is not worth it), otherwise a copy whose rows are padded to a
-    multiple of four elements; the padding is never read."""
+    multiple of four elements; the padding is never read.  An operand that all
+    batches share (batch stride 0, e.g. an expanded view) is copied once and
+    keeps its stride of 0; the size window is about what is physically there."""
     l, r, c = T.shape
+    shared = stride == 0 and l > 1
+    physical = r * c if shared else T.numel()
     if (T.data_ptr() % 16 == 0 and ld % 4 == 0 and stride % 4 == 0) or \
-            not ALIGN_COPY_MIN <= T.numel() <= ALIGN_COPY_MAX:
+            not ALIGN_COPY_MIN <= physical <= ALIGN_COPY_MAX:
         return T, trans, ld, stride
+    src = T[:1] if shared else T
     inner, outer = (c, r) if trans == 0 else (r, c)
     ldp = (inner + 3) // 4 * 4
-    buf = torch.empty(l, outer, ldp, dtype=T.dtype, device=T.device)
+    buf = torch.empty(src.shape[0], outer, ldp, dtype=T.dtype, device=T.device)
     if trans == 0:
         view = buf[..., :c]
-        view.copy_(T)
+        view.copy_(src)
     else:
         view = buf[..., :r].transpose(1, 2)
-        view.copy_(T)
+        view.copy_(src)
+    if shared:
+        return view.expand(l, r, c), trans, ldp, 0
     return view, trans, ldp, outer * ldp
 
 

@@ -144,7 +144,9 @@ int cmk_min_bmm_f32(const float* A, const float* B,
  * allocates and frees nothing.  Problems whose cmk_workspace_bytes() exceeds
  * that size are refused with CMK_ERR_WORKSPACE.  All calls on one GPU share
  * the array: calls that may overlap on one GPU (different streams) race and
- * must be serialised by the caller.  No counterpart in the reference, which
+ * must be serialised by the caller.  The first call on a device looks up the
+ * array's address, which is not a stream operation: make one call outside any
+ * graph capture before capturing it.  No counterpart in the reference, which
  * allocates through PyTorch at every call (minbmm.py:116-122).
  */
 #define CMK_STATIC_SCRATCH_BYTES (4u << 20)
@@ -177,7 +179,10 @@ int cmk_topk_1d_f32(const float* arr, long long n,
                     void* workspace, size_t workspace_bytes, void* stream);
 
 /* Bytes of device workspace an operation needs (0 = none).  For
- * CMK_OP_TOPK_1D pass the array length in M (L = 1). */
+ * CMK_OP_TOPK_1D pass the array length in M (L = 1).  The work is cut for the
+ * GPU that is current when this is called (its compute-unit count): call it
+ * with the device current on which the operation will be launched, or the
+ * launch may refuse the workspace as too small (CMK_ERR_WORKSPACE). */
 size_t cmk_workspace_bytes(int op, int L, int M, int N, int K, int dim);
 
 /* Message describing the last failure on the calling thread ("" if none). */

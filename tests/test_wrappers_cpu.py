@@ -161,3 +161,22 @@ def test_unaligned_operands_are_copied_to_padded_rows_when_it_pays():
     # small operands are left alone
     _, _, d = _common.make_desc(torch.zeros(1, 5, 7), torch.zeros(1, 7, 9))
     assert (d.lda, d.ldb) == (7, 9)
+
+
+def test_shared_unaligned_operand_is_copied_once():
+    """An operand that every batch shares (batch stride 0) and that is not 16-byte
+    aligned is copied as one matrix, not once per batch, and keeps its stride of 0."""
+    import torch
+    from custom_matmul_kernels_amd import _common
+    base = torch.arange(300 * 250 + 1, dtype=torch.float32)
+    one = base[1:].view(300, 250)                      # data pointer off by 4 bytes
+    assert one.data_ptr() % 16 != 0
+    T = one[None].expand(8, 300, 250)
+    out, trans, ld, stride = _common._aligned(T, 0, 250, 0)
+    assert (trans, ld, stride) == (0, 252, 0)
+    assert out.shape == T.shape and out.stride(0) == 0 and torch.equal(out, T)
+    assert out.data_ptr() % 16 == 0
+    # the size window looks at what is physically there: a small shared matrix is left alone
+    small = base[1:1 + 40 * 50].view(40, 50)[None].expand(4096, 40, 50)
+    same, _, _, _ = _common._aligned(small, 0, 50, 0)
+    assert same is small

@@ -70,3 +70,42 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit(device):
     fake = ctypes.c_void_p(0x1000)
     assert lib.cmk_min_bmm_f32_static(fake, fake, fake, fake, d, 2, 0, None) == _lib.ERR_WORKSPACE
     assert b"static" in lib.cmk_last_error()
+
+
+def test_static_scratch_entry_point_replays_in_a_hip_graph(device):
+    """After one call outside a capture (the first call on a device looks up the
+    scratch array's address, which is not a stream operation) the entry point is
+    kernel launches only: captured once, every replay with new inputs matches the
+    eager workspace entry point."""
+    lib = _lib.load()
+    L, M, N, K, dim = 1, 2048, 4096, 64, 2
+    assert 0 < lib.cmk_workspace_bytes(_lib.OP_MIN_BMM, L, M, N, K, dim) <= STATIC_SCRATCH_BYTES
+    print("static scratch under graph capture", (L, M, N, K), flush=True)
+    A, B = seeded(L, M, N, K, seed=77)
+    Ad, Bd = A.to(device), B.to(device)
+    d = _desc(Ad, Bd)
+    values = torch.empty([L, M], device=device)
+    indices = torch.empty([L, M], device=device, dtype=torch.int64)
+
+    def enqueue():
+        stream = torch.cuda.current_stream(device).cuda_stream
+        _lib.check(lib.cmk_min_bmm_f32_static(Ad.data_ptr(), Bd.data_ptr(), values.data_ptr(),
+                                              indices.data_ptr(), d, dim, 0, stream))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        enqueue()                                       # the warm-up call, outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue()
+    gen = torch.Generator().manual_seed(5)
+    for step in range(3):
+        Ad.copy_(torch.randn(L, M, K, generator=gen))
+        Bd.copy_(torch.randn(L, K, N, generator=gen))
+        graph.replay()
+        torch.cuda.synchronize()
+        got_v, got_i = values.clone(), indices.clone()
+        want_v, want_i = _run(lib, Ad, Bd, dim, static=False)   # eager, between the replays
+        assert torch.equal(got_v, want_v) and torch.equal(got_i, want_i), "replay %d differs" % step
