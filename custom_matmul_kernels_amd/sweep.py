@@ -143,6 +143,28 @@ def write_csv(rows, path):
         w.writerows(rows)
 
 
+def write_table(rows, path, command=None):
+    """A compact text table: one line per size, per variant its milliseconds per
+    call and the MiB its results occupy."""
+    names = []
+    for r in rows:
+        if r["variant"] not in names:
+            names.append(r["variant"])
+    r0 = rows[0]
+    with open(path, "w") as f:
+        f.write("%s  A[%d,N,%d] @ B[%d,%d,N]: ms per call | MiB held by the results (the product C counts "
+                "for the unfused variants)\n" % (r0["op"], r0["l"], r0["k"], r0["l"], r0["k"]))
+        if command:
+            f.write("command: %s\n" % command)
+        f.write("%8s" % "N" + "".join("  %28s" % n for n in names) + "\n")
+        for n in sorted({r["n"] for r in rows}):
+            line = "%8d" % n
+            for name in names:
+                sel = [r for r in rows if r["n"] == n and r["variant"] == name]
+                line += "  %14.4f | %11.2f" % (sel[0]["ms"], sel[0]["result_mib"]) if sel else " " * 30
+            f.write(line + "\n")
+
+
 def plot(rows, path, quantity="ms"):
     """One line per variant, N on the x axis (the notebooks' figure)."""
     import matplotlib
@@ -179,6 +201,7 @@ def main(argv=None):
     ap.add_argument("--topk", type=int, default=128)
     ap.add_argument("--dim", type=int, default=2)
     ap.add_argument("--csv", default=None)
+    ap.add_argument("--table", default=None, help="write a compact text table (ms and result MiB per variant)")
     ap.add_argument("--plot", default=None)
     ap.add_argument("--plot-quantity", choices=("ms", "tflops", "result_mib", "peak_mib"), default="ms")
     a = ap.parse_args(argv)
@@ -186,6 +209,8 @@ def main(argv=None):
                out=sys.stdout)
     if a.csv:
         write_csv(rows, a.csv)
+    if a.table:
+        write_table(rows, a.table, "python -m custom_matmul_kernels_amd.sweep " + " ".join(argv if argv is not None else sys.argv[1:]))
     if a.plot:
         plot(rows, a.plot, a.plot_quantity)
     return 0
