@@ -133,9 +133,22 @@ def make_workloads(torch, cmk, O, dev):
 
     W = {}
 
-    def min_wl(name, L, M, N, K, dim=2, distance="inner", cpu_rows=None, config=None):
+    def min_wl(name, L, M, N, K, dim=2, distance="inner", cpu_rows=None, config=None, screen=True):
+        """`screen` False keeps squared l2 on the vector unit whatever the size (the
+        operator's own choice is by size; both routes return the same bits)."""
+        import custom_matmul_kernels_amd.minbmm as minbmm
         op = cmk.MinBMMCUDA(distance=distance)
         inner = distance == "inner"
+        on_matrix_pipe = inner or (distance == "l2" and screen and L * M * N * K >= minbmm.L2_SCREEN_MIN_WORK)
+
+        def run(A, B):
+            if distance == "l2" and not screen:
+                keep, minbmm.L2_SCREEN_MIN_WORK = minbmm.L2_SCREEN_MIN_WORK, 1 << 62
+                try:
+                    return op(A, B, dim=dim)
+                finally:
+                    minbmm.L2_SCREEN_MIN_WORK = keep
+            return op(A, B, dim=dim)
 
         def make():
             A, B = randn_pair(L, M, N, K)
@@ -159,11 +172,15 @@ def make_workloads(torch, cmk, O, dev):
             assert torch.equal(vs, torch.from_numpy(cv)) and torch.equal(is_, torch.from_numpy(ci).long())
             return "%d of %d output rows bit-equal to the C oracle's %s accumulation" % (len(rows), kept, distance)
 
-        per = 2.0 if inner else (3.0 if distance == "l2" else 2.0)
-        w = dict(make=make, run=lambda A, B: op(A, B, dim=dim), flop=per * L * M * N * K, parity=parity,
+        # flop: what the route executes per product term (matrix pipe: multiply + add of the
+        # screening product; vector unit: subtract, multiply, add for l2, subtract, |.|, add for l1 counted as 2)
+        per = 2.0 if on_matrix_pipe else (3.0 if distance == "l2" else 2.0)
+        w = dict(make=make, run=run, flop=per * L * M * N * K, parity=parity,
                  desc="min_bmm%s fp32 A[%d,%d,%d] @ B[%d,%d,%d], min+argmin over dim=%d" % (
-                     "" if inner else " distance=" + distance, L, M, K, L, K, N, dim))
-        if not inner:
+                     "" if inner else " distance=" + distance + (
+                         " (screened on the matrix pipe, settled exactly)" if on_matrix_pipe else " (vector unit)"),
+                     L, M, K, L, K, N, dim))
+        if not on_matrix_pipe:
             w["valu_ops"] = 2.0 * L * M * N * K   # subtract + fused multiply-add, or subtract + add of |.|
         if cpu_rows:
             w.update(cpu=lambda A, B, r0: torch.bmm(A[:, r0:r0 + cpu_rows], B).min(-1), cpu_rows=cpu_rows, rows=M,
@@ -318,6 +335,7 @@ def make_workloads(torch, cmk, O, dev):
     masks_wl("derive_masks", 128, 1024, 1024)
     masks_wl("derive_masks_4GiB", 1024, 2048, 2048)
     min_wl("min_bmm_l2", 1, 16384, 16384, 256, distance="l2")
+    min_wl("min_bmm_l2_vector", 1, 16384, 16384, 256, distance="l2", screen=False)
     min_wl("min_bmm_l1", 1, 16384, 16384, 256, distance="l1")
     # the shapes the reference publishes numbers for (its notebooks' printed results and plots, Tesla T4)
     bmm_wl("ref_bmm_8192x512", 1, 8192, 8192, 512)             # colab/test_bmm.ipynb:2163-2164

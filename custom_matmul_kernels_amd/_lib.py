@@ -16,7 +16,7 @@ CSRC_DIR = os.path.join(_HERE, "csrc")
 
 ABI_VERSION = 1
 
-OP_BMM, OP_MBMM, OP_MIN_BMM, OP_TOPK_BMM, OP_TOPK_1D = range(5)
+OP_BMM, OP_MBMM, OP_MIN_BMM, OP_TOPK_BMM, OP_TOPK_1D, OP_MIN_BMM_L2 = range(6)
 DIST_INNER, DIST_L2, DIST_L1 = range(3)
 ERR_INVALID_ARG, ERR_UNSUPPORTED, ERR_WORKSPACE = -1, -2, -3
 

@@ -62,6 +62,7 @@ int compute_units() {
 
 size_t bmm_workspace_bytes(int L, int M, int N, int K);
 size_t min_workspace_bytes(int L, int Xext, int Yext, int K);
+size_t min_l2_workspace_bytes(int L, int Xext, int Yext, int K);
 size_t topk_workspace_bytes(int L, int Xext, int Yext, int K);
 size_t topk1d_workspace_bytes(long long n);
 
@@ -75,6 +76,9 @@ extern "C" size_t cmk_workspace_bytes(int op, int L, int M, int N, int K, int di
     case CMK_OP_MIN_BMM:
       if (dim != 1 && dim != 2) return 0;
       return cmk::min_workspace_bytes(L, dim == 2 ? N : M, dim == 2 ? M : N, K);
+    case CMK_OP_MIN_BMM_L2:
+      if (dim != 1 && dim != 2) return 0;
+      return cmk::min_l2_workspace_bytes(L, dim == 2 ? N : M, dim == 2 ? M : N, K);
     case CMK_OP_TOPK_BMM:
       if (dim != 1 && dim != 2) return 0;
       return cmk::topk_workspace_bytes(L, dim == 2 ? N : M, dim == 2 ? M : N, K);

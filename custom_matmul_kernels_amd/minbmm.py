@@ -4,6 +4,12 @@ import torch
 from . import _common, _lib
 
 
+# Squared l2 goes through the matrix pipe (screening there, exact evaluation of
+# the surviving candidates, bit-equal results) from this many multiply-adds
+# L*m*n*k on; below, the extra launches cost more than the vector route saves.
+L2_SCREEN_MIN_WORK = 1 << 28
+
+
 class MinBMMCUDA:
     """Drop-in for the reference's ``MinBMMCUDA`` (reference minbmm.py:7-148):
     same constructor keywords, same ``__call__(A, B, dim=1)`` returning
@@ -41,7 +47,12 @@ class MinBMMCUDA:
         indices = torch.empty([l, kept], device=A.device, dtype=torch.int64)
         if values.numel():
             A2, B2, desc = _common.make_desc(A, B)
-            ws, ws_bytes = _common.workspace(_lib.OP_MIN_BMM, l, m, n, k, dim, A.device)
+            op = _lib.OP_MIN_BMM
+            if self.distance == "l2" and l * m * n * k >= L2_SCREEN_MIN_WORK:
+                op = _lib.OP_MIN_BMM_L2
+            ws, ws_bytes = _common.workspace(op, l, m, n, k, dim, A.device)
+            if op == _lib.OP_MIN_BMM_L2 and ws is None:   # shape outside the screening route
+                ws, ws_bytes = _common.workspace(_lib.OP_MIN_BMM, l, m, n, k, dim, A.device)
             with torch.cuda.device(A.device):
                 _lib.check(self._lib.cmk_min_bmm_f32(
                     A2.data_ptr(), B2.data_ptr(), values.data_ptr(), indices.data_ptr(), desc,
