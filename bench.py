@@ -139,7 +139,7 @@ def make_workloads(torch, cmk, O, dev):
         import custom_matmul_kernels_amd.minbmm as minbmm
         op = cmk.MinBMMCUDA(distance=distance)
         inner = distance == "inner"
-        on_matrix_pipe = inner or (distance == "l2" and screen and L * M * N * K >= minbmm.L2_SCREEN_MIN_WORK)
+        on_matrix_pipe = inner or (distance == "l2" and screen and minbmm.screens_l2(L, M, N, K))
 
         def run(A, B):
             if distance == "l2" and not screen:

@@ -116,12 +116,13 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     }
-    core.template tile<kInner, !MASKED>(X, Y, lds, acc);
-
     // A kept tile whose masks can be fetched with 16-byte loads gets them staged
-    // in LDS (the operand buffers are free by now): 128 rows of 128 element-mask
-    // bytes, then the tile's 16x16 thread-mask bytes.
+    // in LDS: 128 rows of 128 element-mask bytes, then the tile's 16x16
+    // thread-mask bytes.  They are requested before the product starts, so that
+    // they arrive while it runs, and go to LDS once the operand buffers are free.
     bool staged = false;
+    f32x4 mask_regs[4];
+    uint8_t tmask_reg = 0;
     if constexpr (MASKED) {
       const int m0 = (tile_m0 + ti) * C::TX;
       staged = m0 + 128 <= a.M && n0 + 128 <= a.N && (a.N & 15) == 0 &&
@@ -129,22 +130,33 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
       if (staged) {
         typedef const f32x4 __attribute__((address_space(1))) * g16p;
         typedef const uint8_t __attribute__((address_space(1))) * g1p;
-        core.wait_loads();
-        __syncthreads();  // nobody reads operand fragments any more
-        uint8_t* ml = reinterpret_cast<uint8_t*>(lds);
         const uint8_t* eb = a.element_mask + (mb * a.M + m0) * a.N + n0;
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
           const int idx = threadIdx.x + kThreads * p;
           const int row = idx >> 3, c16 = (idx & 7) * 16;
-          const f32x4 v = *(g16p)(eb + (long long)row * a.N + c16);
-          *reinterpret_cast<f32x4*>(ml + row * kMaskPitch + c16) = v;
+          mask_regs[p] = *(g16p)(eb + (long long)row * a.N + c16);
         }
         const int tn8 = (a.N + 7) >> 3;
         const int tm8 = (a.M + 7) >> 3;
-        ml[kMaskRows * kMaskPitch + threadIdx.x] =
-            *(g1p)(a.thread_mask + (mb * tm8 + (m0 >> 3) + (threadIdx.x >> 4)) * tn8 + (n0 >> 3) +
-                   (threadIdx.x & 15));
+        tmask_reg = *(g1p)(a.thread_mask + (mb * tm8 + (m0 >> 3) + (threadIdx.x >> 4)) * tn8 + (n0 >> 3) +
+                           (threadIdx.x & 15));
+      }
+    }
+    core.template tile<kInner, !MASKED>(X, Y, lds, acc);
+
+    if constexpr (MASKED) {
+      if (staged) {
+        core.wait_loads();
+        __syncthreads();  // nobody reads operand fragments any more
+        uint8_t* ml = reinterpret_cast<uint8_t*>(lds);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          const int idx = threadIdx.x + kThreads * p;
+          const int row = idx >> 3, c16 = (idx & 7) * 16;
+          *reinterpret_cast<f32x4*>(ml + row * kMaskPitch + c16) = mask_regs[p];
+        }
+        ml[kMaskRows * kMaskPitch + threadIdx.x] = tmask_reg;
         __syncthreads();
       }
     }

@@ -7,7 +7,15 @@ from . import _common, _lib
 # Squared l2 goes through the matrix pipe (screening there, exact evaluation of
 # the surviving candidates, bit-equal results) from this many multiply-adds
 # L*m*n*k on; below, the extra launches cost more than the vector route saves.
-L2_SCREEN_MIN_WORK = 1 << 28
+# Measured on MI355X: the screening route takes 0.034 ms at least, the vector
+# route 0.025 ms at k = 16 and 0.042 ms at k = 64 for 2^26 multiply-adds.
+L2_SCREEN_MIN_WORK = 1 << 26
+
+
+def screens_l2(l, m, n, k):
+    """Whether MinBMMCUDA(distance="l2") takes the matrix pipe for this shape."""
+    work = l * m * n * k
+    return work >= L2_SCREEN_MIN_WORK and (k >= 48 or work >= 4 * L2_SCREEN_MIN_WORK)
 
 
 class MinBMMCUDA:
@@ -48,7 +56,7 @@ class MinBMMCUDA:
         if values.numel():
             A2, B2, desc = _common.make_desc(A, B)
             op = _lib.OP_MIN_BMM
-            if self.distance == "l2" and l * m * n * k >= L2_SCREEN_MIN_WORK:
+            if self._distance == _lib.DIST_L2 and screens_l2(l, m, n, k):
                 op = _lib.OP_MIN_BMM_L2
             ws, ws_bytes = _common.workspace(op, l, m, n, k, dim, A.device)
             if op == _lib.OP_MIN_BMM_L2 and ws is None:   # shape outside the screening route
