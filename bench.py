@@ -504,6 +504,7 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="min_bmm_large")
+    ap.add_argument("--details", default=None, help="also write the full record (one JSON line) to this file")
     ap.add_argument("--no-others", action="store_true", help="skip the short runs of the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--no-parity", action="store_true", help="skip the parity checks")
@@ -613,13 +614,13 @@ def main():
             del cpu_args, dev_args
             torch.cuda.empty_cache()
         out["other_workloads"] = others
-    # The full record goes to stderr (and to gpurun_out/ when that exists); the one
+    # The full record goes to stderr (and to the file --details names); the one
     # line on stdout keeps the headline in full and, per other workload, the
     # figures only, so that it stays a few kilobytes.
     full = json.dumps(out)
     print(full, file=sys.stderr)
-    if os.path.isdir(os.path.join(ROOT, "gpurun_out")):
-        with open(os.path.join(ROOT, "gpurun_out", "bench_details.json"), "w") as f:
+    if a.details:
+        with open(a.details, "w") as f:
             f.write(full + "\n")
     if "other_workloads" in out:
         keep = ("config", "kernel_ms", "kernel_ms_median", "frac_fp32_mfma_peak", "frac_fp32_mfma_peak_region_average",
