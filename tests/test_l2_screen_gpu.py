@@ -176,3 +176,54 @@ def test_default_threshold_uses_the_screening_for_large_problems(device):
     cols = np.linspace(0, 8191, 32).astype(np.int64)
     cv, ci = O.c_min_bmm(A.numpy(), np.ascontiguousarray(B.numpy()[:, :, cols]), 1, 1)
     same((v.cpu()[:, cols], i.cpu()[:, cols]), (torch.from_numpy(cv), torch.from_numpy(ci).long()))
+
+
+def _sweep_case(rng):
+    L = int(rng.choice([1, 1, 2, 3]))
+    M = int(rng.integers(1, 700))
+    N = int(rng.integers(1, 700))
+    K = int(rng.choice([1, 2, 7, 16, 31, 64, 100, 257, 420]))
+    kind = rng.choice(["normal", "clustered", "integers", "offset", "scales", "sparse"])
+    g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+    if kind == "normal":
+        A, B = torch.randn(L, M, K, generator=g), torch.randn(L, K, N, generator=g)
+    elif kind == "clustered":
+        # a handful of centres, points are centres plus noise at the rounding level: near ties everywhere
+        C = torch.randn(L, 5, K, generator=g)
+        ia = torch.randint(0, 5, (L, M), generator=g)
+        ib = torch.randint(0, 5, (L, N), generator=g)
+        A = torch.gather(C, 1, ia[..., None].expand(L, M, K)) + 1e-6 * torch.randn(L, M, K, generator=g)
+        B = (torch.gather(C, 1, ib[..., None].expand(L, N, K)) + 1e-6 * torch.randn(L, N, K, generator=g)).transpose(1, 2)
+    elif kind == "integers":
+        A = torch.randint(-3, 4, (L, M, K), generator=g).float()
+        B = torch.randint(-3, 4, (L, K, N), generator=g).float()
+    elif kind == "offset":
+        off = float(rng.choice([10.0, 300.0, 1e4]))
+        A = off + torch.randn(L, M, K, generator=g)
+        B = off + torch.randn(L, K, N, generator=g)
+    elif kind == "scales":
+        A = torch.randn(L, M, K, generator=g) * 10.0 ** torch.randint(-6, 7, (L, M, 1), generator=g).float()
+        B = torch.randn(L, K, N, generator=g) * 10.0 ** torch.randint(-6, 7, (L, 1, N), generator=g).float()
+    else:
+        A = torch.randn(L, M, K, generator=g) * (torch.rand(L, M, K, generator=g) < 0.1)
+        B = torch.randn(L, K, N, generator=g) * (torch.rand(L, K, N, generator=g) < 0.1)
+    return kind, A.contiguous(), B.contiguous()
+
+
+def test_screened_l2_seeded_sweep_over_shapes_and_data(device, monkeypatch):
+    """Sixty seeded cases over shapes, layouts, axes and kinds of data that stress
+    the screen in different ways (near ties, exact ties, cancellation, mixed
+    magnitudes, many zeros): both routes return the same bits, and the oracle
+    agrees on every fourth case."""
+    rng = np.random.default_rng(2024)
+    for case in range(60):
+        kind, A, B = _sweep_case(rng)
+        mode = str(rng.choice(["nn", "tt", "nt", "tn"]))
+        dim = int(rng.choice([1, 2]))
+        say("sweep", case, kind, tuple(A.shape), tuple(B.shape), mode, dim)
+        Ad, Bd = place(A, B, mode, device)
+        vec, scr = both_routes(monkeypatch, Ad, Bd, dim)
+        same(scr, vec)
+        if case % 4 == 0:
+            cv, ci = O.c_min_bmm(A.numpy(), B.numpy(), dim, 1)
+            same(scr, (torch.from_numpy(cv), torch.from_numpy(ci).long()))
