@@ -227,3 +227,27 @@ def test_screened_l2_seeded_sweep_over_shapes_and_data(device, monkeypatch):
         if case % 4 == 0:
             cv, ci = O.c_min_bmm(A.numpy(), B.numpy(), dim, 1)
             same(scr, (torch.from_numpy(cv), torch.from_numpy(ci).long()))
+
+
+def test_screened_l2_on_strided_views_and_a_shared_operand(device, monkeypatch):
+    """Operands that are windows of wider tensors (leading dimension beyond the
+    row length, consumed in place) and an operand shared by all batches (batch
+    stride 0)."""
+    say("views")
+    g = torch.Generator().manual_seed(31)
+    wideA = torch.randn(3, 260, 96, generator=g)
+    wideB = torch.randn(3, 80, 400, generator=g)
+    A, B = wideA[:, 4:250, 8:72], wideB[:, 16:80, 40:360]          # [3,246,64] and [3,64,320]
+    Ad, Bd = wideA.to(device)[:, 4:250, 8:72], wideB.to(device)[:, 16:80, 40:360]
+    for dim in (1, 2):
+        vec, scr = both_routes(monkeypatch, Ad, Bd, dim)
+        same(scr, vec)
+        cv, ci = O.c_min_bmm(A.contiguous().numpy(), B.contiguous().numpy(), dim, 1)
+        same(scr, (torch.from_numpy(cv), torch.from_numpy(ci).long()))
+    shared = wideB[:1, 16:80, 40:360]
+    Bs = shared.to(device).expand(3, -1, -1)
+    for dim in (1, 2):
+        vec, scr = both_routes(monkeypatch, Ad, Bs, dim)
+        same(scr, vec)
+        cv, ci = O.c_min_bmm(A.contiguous().numpy(), shared.expand(3, -1, -1).contiguous().numpy(), dim, 1)
+        same(scr, (torch.from_numpy(cv), torch.from_numpy(ci).long()))
