@@ -251,3 +251,44 @@ def test_screened_l2_on_strided_views_and_a_shared_operand(device, monkeypatch):
         same(scr, vec)
         cv, ci = O.c_min_bmm(A.contiguous().numpy(), shared.expand(3, -1, -1).contiguous().numpy(), dim, 1)
         same(scr, (torch.from_numpy(cv), torch.from_numpy(ci).long()))
+
+
+def test_screened_l2_replays_in_a_hip_graph(device, monkeypatch):
+    """The screening route is kernel launches only (its counter is cleared by its
+    first kernel): captured once, every replay on new inputs - one of them with
+    duplicated points, so that rows are queued - equals the eager vector route."""
+    say("graph replay")
+    monkeypatch.setattr(minbmm, "L2_SCREEN_MIN_WORK", 0)
+    L, M, N, K = 2, 300, 520, 72
+    gen = torch.Generator().manual_seed(41)
+    A = torch.randn(L, M, K, generator=gen).to(device)
+    B = torch.randn(L, K, N, generator=gen).to(device)
+    op = MinBMMCUDA(distance="l2")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            op(A, B, dim=2)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = op(A, B, dim=2)
+    for step in range(3):
+        a = torch.randn(L, M, K, generator=gen)
+        b = torch.randn(L, K, N, generator=gen)
+        if step == 1:
+            b[:, :, 100] = b[:, :, 7]
+            b[:, :, 300] = b[:, :, 7]
+            a[:, 5] = b[:, :, 7]
+        A.copy_(a)
+        B.copy_(b)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        monkeypatch.setattr(minbmm, "L2_SCREEN_MIN_WORK", 1 << 62)
+        want = op(A, B, dim=2)
+        monkeypatch.setattr(minbmm, "L2_SCREEN_MIN_WORK", 0)
+        torch.cuda.synchronize()
+        same((got[0].cpu(), got[1].cpu()), (want[0].cpu(), want[1].cpu()))
+        if step == 1:
+            assert int(got[1][0, 5]) == 7
