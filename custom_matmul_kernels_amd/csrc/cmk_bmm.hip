@@ -35,7 +35,15 @@ constexpr int kMaskPitch = 144;   // ... of 128 bytes, 16-byte aligned, skewed o
 // for products with too few 128x128 tiles to occupy the chip (dense only).
 template <int XK, int YK, bool MASKED, int B = 2>
 __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
-  using C = Core<XK, YK, 2, 2, B, B>;
+  // In the masked product a lane's two accumulators of one row are neighbouring
+  // columns (Y_PAIRS): C leaves as 8-byte stores, the two element-mask bytes come
+  // with one LDS read and share a thread-mask byte (3 % faster on the masked
+  // shapes; the dense product measured 3 % slower with it and keeps its columns
+  // 32 apart).
+  constexpr bool PAIRS = B == 2 && MASKED;
+  using C = Core<XK, YK, 2, 2, B, B, 32, kReadsPaired, false, false, true, PAIRS>;
+  // column of block `by` of this lane within the wave's columns
+  auto col_of = [](int by, int l32) { return PAIRS ? 2 * l32 + by : by * 32 + l32; };
   static_assert(B == 2 || !MASKED, "the masks are laid out for 128x128 tiles");
   __shared__ __attribute__((aligned(16))) float lds[C::ldsFloats];
 
@@ -171,40 +179,52 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
       // interior: row addresses are scalar, the lane part is one 32-bit offset
       typedef float __attribute__((address_space(1))) * gfp;
       typedef const uint8_t __attribute__((address_space(1))) * gbp;
+      typedef f32x2 __attribute__((address_space(1))) * gf2p;
       char* base = reinterpret_cast<char*>(uniform_ptr(Cb + (long long)mw * a.N + nw));
-      const unsigned voff = static_cast<unsigned>((4 * half * a.N + l32) * 4);
+      const unsigned voff = static_cast<unsigned>((4 * half * a.N + col_of(0, l32)) * 4);
+      constexpr int kByStep = PAIRS ? 4 : 128;   // bytes from block by = 0 to by = 1
+      // both accumulators of a row in one store: rows of C must stay 8-byte aligned
+      const bool pair_store = PAIRS && (a.N & 1) == 0 && (reinterpret_cast<uintptr_t>(Cb) & 7) == 0;
+      auto put = [&](char* rp, float v0, float v1) {
+        if (pair_store) {
+          __builtin_nontemporal_store(f32x2{v0, v1}, (gf2p)(rp + voff));
+        } else {
+          __builtin_nontemporal_store(v0, (gfp)(rp + voff));
+          __builtin_nontemporal_store(v1, (gfp)(rp + voff + kByStep));
+        }
+      };
       if constexpr (!MASKED) {
 #pragma unroll
         for (int bx = 0; bx < B; ++bx)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             char* rp = base + (long long)(bx * 32 + 8 * (r >> 2) + (r & 3)) * a.N * 4;
-#pragma unroll
-            for (int by = 0; by < B; ++by) __builtin_nontemporal_store(acc[bx][by][r], (gfp)(rp + voff + by * 128));
+            if constexpr (B == 2) {
+              put(rp, acc[bx][0][r], acc[bx][1][r]);
+            } else {
+              __builtin_nontemporal_store(acc[bx][0][r], (gfp)(rp + voff));
+            }
           }
       } else if (staged) {
         // masks come from LDS: byte reads there cost no vector-memory instructions
         const uint8_t* ml = reinterpret_cast<const uint8_t*>(lds);
         const int mwl = (wv % 2) * 64, nwl = (wv / 2) * 64;
-        const uint8_t* tl = ml + kMaskRows * kMaskPitch + (mwl >> 3) * 16 + (nwl >> 3) + (l32 >> 3);
-        const uint8_t* el = ml + (mwl + 4 * half) * kMaskPitch + nwl + l32;
+        // (the lane's two columns 2 * l32 and 2 * l32 + 1 share a micro-tile and are
+        // two neighbouring element-mask bytes)
+        const uint8_t* tl = ml + kMaskRows * kMaskPitch + (mwl >> 3) * 16 + (nwl >> 3) + (l32 >> 2);
+        const uint8_t* el = ml + (mwl + 4 * half) * kMaskPitch + nwl + 2 * l32;
 #pragma unroll
         for (int bx = 0; bx < 2; ++bx)
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            uint8_t tmk[2];
-#pragma unroll
-            for (int by = 0; by < 2; ++by) tmk[by] = tl[(bx * 4 + q) * 16 + by * 4];
+            const uint8_t tmk = tl[(bx * 4 + q) * 16];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int r = 4 * q + e;
               const int rowc = bx * 32 + 8 * q + e;
               char* rp = base + (long long)rowc * a.N * 4;
-#pragma unroll
-              for (int by = 0; by < 2; ++by) {
-                const uint8_t em = el[rowc * kMaskPitch + by * 32];
-                __builtin_nontemporal_store(tmk[by] ? acc[bx][by][r] * (float)em : 0.f, (gfp)(rp + voff + by * 128));
-              }
+              const unsigned em2 = *reinterpret_cast<const uint16_t*>(el + rowc * kMaskPitch);
+              put(rp, tmk ? acc[bx][0][r] * (float)(em2 & 0xffu) : 0.f, tmk ? acc[bx][1][r] * (float)(em2 >> 8) : 0.f);
             }
           }
       } else {
@@ -212,27 +232,21 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
         const int tm8 = (a.M + 7) >> 3;
         const uint8_t* eb = uniform_ptr(a.element_mask + (mb * a.M + mw) * a.N + nw);
         const uint8_t* tb = uniform_ptr(a.thread_mask + (mb * tm8 + (mw >> 3)) * tn8 + (nw >> 3));
-        const unsigned eoff = static_cast<unsigned>(4 * half * a.N + l32);
-        const unsigned toff = static_cast<unsigned>(l32 >> 3);
+        const unsigned eoff = static_cast<unsigned>(4 * half * a.N + 2 * l32);
+        const unsigned toff = static_cast<unsigned>(l32 >> 2);
 #pragma unroll
         for (int bx = 0; bx < 2; ++bx)
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            uint8_t tmk[2];
-#pragma unroll
-            for (int by = 0; by < 2; ++by)
-              tmk[by] = *(gbp)(tb + (long long)(bx * 4 + q) * tn8 + toff + by * 4);
+            const uint8_t tmk = *(gbp)(tb + (long long)(bx * 4 + q) * tn8 + toff);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int r = 4 * q + e;
               const long long rowc = bx * 32 + 8 * q + e;
               char* rp = base + rowc * a.N * 4;
               const uint8_t* ep = eb + rowc * a.N;
-#pragma unroll
-              for (int by = 0; by < 2; ++by) {
-                const uint8_t em = *(gbp)(ep + eoff + by * 32);
-                __builtin_nontemporal_store(tmk[by] ? acc[bx][by][r] * (float)em : 0.f, (gfp)(rp + voff + by * 128));
-              }
+              const uint8_t em0 = *(gbp)(ep + eoff), em1 = *(gbp)(ep + eoff + 1);
+              put(rp, tmk ? acc[bx][0][r] * (float)em0 : 0.f, tmk ? acc[bx][1][r] * (float)em1 : 0.f);
             }
           }
       }
@@ -241,7 +255,7 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
       for (int bx = 0; bx < B; ++bx) {
 #pragma unroll
         for (int by = 0; by < B; ++by) {
-          const int n = nw + by * 32 + l32;
+          const int n = nw + col_of(by, l32);
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int m = mw + bx * 32 + acc_row(r, half);

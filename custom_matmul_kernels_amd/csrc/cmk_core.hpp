@@ -41,6 +41,7 @@
 namespace cmk {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // Operands live in global memory; loading through pointers that say so gives
@@ -253,9 +254,16 @@ constexpr int kReadsSingle = 2;   // four single reads with immediate offsets
 // ADDR_REGS keeps every fragment address in a register of its own for the whole
 // sequence (no vector arithmetic in the slab loop); without it the compiler is
 // free to re-derive them, which a kernel short of registers prefers.
+//
+// Y_PAIRS (BY == 2) deals the Y rows of a wave to its two blocks alternately -
+// block b of lane l takes row 2 * (l % 32) + b of the wave's 64 instead of
+// (l % 32) + 32 * b - so that a lane's two accumulators of one X row are
+// neighbours along Y: an epilogue that stores along Y writes them as one
+// 8-byte store.  Only the fragment addresses change.
 template <int XK, int YK, int WX, int WY, int BX, int BY, int KS_ = 32, int RC_READS = kReadsPaired,
-          bool STAGGER = false, bool Y_ONCE = false, bool ADDR_REGS = true>
+          bool STAGGER = false, bool Y_ONCE = false, bool ADDR_REGS = true, bool Y_PAIRS = false>
 struct Core {
+  static_assert(!Y_PAIRS || BY == 2, "Y_PAIRS pairs the two Y blocks of a wave");
   static_assert(WX * WY == 4 || WX * WY == 8 || WX * WY == 16, "4, 8 or 16 waves per work-group");
   static constexpr int NT = WX * WY * 64;      // threads per work-group
   static constexpr int KS = KS_;
@@ -451,7 +459,7 @@ struct Core {
       for (int b = 0; b < BY; ++b)
 #pragma unroll
         for (int g = 0; g < NAY; ++g) {
-          const int row = yr + 32 * b;
+          const int row = Y_PAIRS ? (wave / WX) * BY * 32 + 2 * (lane & 31) + b : yr + 32 * b;
           yad[b][g] = base + 4u * (YK == KC ? lds_pos<KC, TY, KS>(row, g * 8 + half * 4) : half * 4 * TY + row);
           if (ADDR_REGS) asm volatile("" : "+v"(yad[b][g]));
         }
@@ -550,6 +558,7 @@ struct Core {
                                              f32x16 (&acc)[BX][BY]) {
     const int l32 = tid & 31;
     const int xw = ((tid >> 6) % WX) * BX * 32 + 4 * half;   // first X row of this half-wave
+    static_assert(!Y_PAIRS, "the vector-unit distances deal Y rows block by block");
     const int yl = ((tid >> 6) / WX) * BY * 32 + l32;        // this lane's first Y row
     float y[BY][8];
 #pragma unroll
