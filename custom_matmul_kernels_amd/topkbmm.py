@@ -4,6 +4,27 @@ import torch
 from . import _common, _lib
 
 
+# The vector-unit distance kernels of top-k run 40 % faster when the operand of
+# the reduced axis is stored with that axis contiguous (its points are then LDS
+# columns that a half-wave reads as broadcasts without extra address registers;
+# the other form spills at the kernel's 128 registers per lane).  From this many
+# multiply-adds on, an operand stored the other way is copied once: the copy
+# moves the operand, the kernel does l*m*n*k vector operations on it.
+DIST_RELAYOUT_MIN_WORK = 1 << 24
+
+
+def _reduced_axis_contiguous(A, B, dim):
+    """A[l,m,k], B[l,k,n] with the operand of the reduced axis (A for dim 1, B for
+    dim 2) stored with that axis contiguous; same values, other strides.  (Copying
+    the other, larger operand into its preferred form as well costs more than the
+    10 % it gives.)"""
+    if dim == 1 and A.stride(-1) == 1 and A.stride(-2) != 1:
+        A = A.transpose(1, 2).contiguous().transpose(1, 2)
+    elif dim == 2 and B.stride(-2) == 1 and B.stride(-1) != 1:
+        B = B.contiguous()
+    return A, B
+
+
 class TopkBMMCUDA:
     """Drop-in for the reference's ``TopkBMMCUDA`` (reference topkbmm.py:7-156):
     same constructor keywords, same ``__call__(A, B, k=128, dim=1)`` returning
@@ -39,6 +60,8 @@ class TopkBMMCUDA:
         values = torch.empty([l, kept, k], device=A.device, dtype=A.dtype)
         indices = torch.empty([l, kept, k], device=A.device, dtype=torch.int64)
         if values.numel():
+            if self._distance != _lib.DIST_INNER and l * m * n * d >= DIST_RELAYOUT_MIN_WORK:
+                A, B = _reduced_axis_contiguous(A, B, dim)
             A2, B2, desc = _common.make_desc(A, B)
             ws, ws_bytes = _common.workspace(_lib.OP_TOPK_BMM, l, m, n, d, dim, A.device)
             with torch.cuda.device(A.device):

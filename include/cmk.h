@@ -53,7 +53,10 @@ extern "C" {
  * vector unit, in the reference's order of operations (d = a - b, then
  * fmaf(d, d, c) or c + fabsf(d), k ascending), a few times slower.
  * cmk_min_bmm_f32 has a second route for L2 that gives the same bits from the
- * matrix pipe (see there). */
+ * matrix pipe (see there).  cmk_topk_bmm_f32 with L2 / L1 runs about 40 % faster
+ * when the operand of the reduced axis is stored with that axis contiguous (A
+ * with transA = 1 for dim 1, B with transB = 0 for dim 2); the Python wrapper
+ * copies a large operand into that form. */
 #define CMK_DIST_INNER 0   /* c += a*b        ("madd")       */
 #define CMK_DIST_L2    1   /* c += (a-b)^2    ("squared_l2") */
 #define CMK_DIST_L1    2   /* c += |a-b|      ("l1")         */
