@@ -74,7 +74,20 @@ __global__ __launch_bounds__(kThreads, 2) void bmm_kernel(BmmArgs a) {
   long long mb = 0;  // batch index into the masks
   if constexpr (MASKED) {
     mb = a.mask_batched ? b : 0;
-    const uint8_t bm = a.block_mask[(mb * a.tiles_m + tile_m0) * a.tiles_n + tile_n];
+    // The work-group's first dependent step.  The byte is the same for all lanes:
+    // it comes through the scalar cache as the aligned word around it (a third of
+    // the latency of a vector byte load), unless that word reaches past the array.
+    const long long bi = (mb * a.tiles_m + tile_m0) * a.tiles_n + tile_n;
+    const long long bytes = (long long)(a.mask_batched ? a.L : 1) * a.tiles_m * a.tiles_n;
+    const uintptr_t at = reinterpret_cast<uintptr_t>(a.block_mask) + bi;
+    uint8_t bm;
+    if ((reinterpret_cast<uintptr_t>(a.block_mask) & 3) == 0 && (bi | 3) < bytes) {
+      typedef const uint32_t __attribute__((address_space(4))) * c32p;
+      const uint32_t word = *(c32p)(at & ~static_cast<uintptr_t>(3));
+      bm = static_cast<uint8_t>(word >> (8 * (at & 3)));
+    } else {
+      bm = a.block_mask[bi];
+    }
     if (bm == 0) {
       // skipped tile: nothing is loaded or multiplied, zeros are written
       const int m0 = tile_m0 * C::TX;
