@@ -60,6 +60,19 @@ def test_workspace_sizes(lib):
     assert w > 0 and w % (1024 * 128 * 8) == 0
     assert lib.cmk_workspace_bytes(_lib.OP_TOPK_1D, 1, 1000, 0, 0, 0) == 128 * 8
     assert lib.cmk_workspace_bytes(_lib.OP_MIN_BMM, 1, 8, 8, 8, 3) == 0   # bad dim
+    # squared l2 on the matrix pipe: norms, the queue, a copy of the reduced-axis operand and
+    # 20 bytes per row and range; always more than the vector route asks for, nothing when K is 0
+    for shape in ((1, 16384, 16384, 256), (1, 4096, 4096, 64), (2, 300, 500, 17)):
+        for dim in (1, 2):
+            small = lib.cmk_workspace_bytes(_lib.OP_MIN_BMM, *shape, dim)
+            big = lib.cmk_workspace_bytes(_lib.OP_MIN_BMM_L2, *shape, dim)
+            assert big > small and big % 256 == 0
+            L, M, N, K = shape
+            x, y = (N, M) if dim == 2 else (M, N)
+            assert big >= 4 * L * (x * K + x + y) + 20 * L * y
+    assert lib.cmk_workspace_bytes(_lib.OP_MIN_BMM_L2, 1, 64, 64, 0, 2) == 0
+    assert lib.cmk_workspace_bytes(_lib.OP_MIN_BMM_L2, 1, 64, 64, 8, 0) == 0
+    assert _lib.OP_MIN_BMM_L2 == 5
 
 
 def _desc(L=1, M=8, N=8, K=8, tA=0, tB=0, lda=None, ldb=None):
